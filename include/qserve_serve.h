@@ -23,6 +23,27 @@ const char* qsv_last_error(void);
 /* x[t] = table[tokens[t]] (float) and h[t] = the same row in the storage type. */
 int qsv_embed(float* x, void* h, const void* table, const int32_t* tokens, int n_tokens, int width, int dtype, void* stream);
 
+/* x[t] = table[tokens[t]] * scale + s(pos[t]),  s(p)[2i] = sin(p freq[i]),  s(p)[2i + 1] = cos(p freq[i])   (float; freq float
+ * [(width + 1) / 2]). */
+int qsv_embed_sinusoid(float* x, const void* table, const int32_t* tokens, const int32_t* pos, const float* freq, float scale,
+                       int n_tokens, int width, int dtype, void* stream);
+/* x[t] += a[t] + (b[t] + c[t]) (each of a, b, c may be NULL); h[t] = x[t] / sqrt(mean(x[t]^2) + eps) * w in the storage type
+ * (h == NULL: the sum only). */
+int qsv_add_rms_norm(float* x, void* h, const void* a, const void* b, const void* c, const void* w, float eps, int n_tokens,
+                     int width, int dtype, void* stream);
+/* out[r] = rms_norm(x[rows[r]]) * w in the storage type (rows == NULL: row r). */
+int qsv_rms_norm_rows(void* out, const float* x, const int32_t* rows, const void* w, float eps, int n_rows, int width, int dtype,
+                      void* stream);
+/* Queries and keys RMS-normed over the whole projection (all heads at once), values optionally blended, cache rows written:
+ *   qf[t, h]         = [ 0 (vdim) | (q[t] / rms(q[t]) * q_w)[h] * scale ]          float [T, heads, vdim + dim]
+ *   pool[g, slot[t]] = [ v'[t, g] | (k[t] / rms(k[t]) * k_w)[g] ]                  [kv_heads, pool_rows, vdim + dim]
+ *   v' = (1 - mix) v + mix v_first[t] if v_first (storage type, rows vf_stride apart, [kv_heads * vdim]) is given, else v.
+ * q, k, v are column ranges of proj (row stride `stride`). */
+int qsv_normed_attention_prep(float* qf, void* pool, int64_t pool_rows, const void* proj, int64_t stride, int q_off, int k_off,
+                              int v_off, int heads, int kv_heads, int dim, int vdim, const void* q_w, const void* k_w, float eps,
+                              float scale, const void* v_first, int64_t vf_stride, float mix, const int64_t* slot, int n_tokens,
+                              int dtype, void* stream);
+
 /* x[t] += layer_norm(y[t]) * w (no bias; variance = mean of squared deviations); h[t] = x[t] in the storage type. */
 int qsv_add_layer_norm(float* x, void* h, const void* y, const void* w, float eps, int n_tokens, int width, int dtype,
                        void* stream);
@@ -52,9 +73,13 @@ int qsv_latent_query(float* qf, const void* q, const void* q_abs, const float* r
  * row(s, j) = block_table[s * table_stride + j / page] * page + j % page.  variant: 0 = default kernel choice.
  * Several pools in one launch: heads [g * heads_per_pool, (g + 1) * heads_per_pool) read the pool that starts pool_stride
  * elements after pool g - 1 (one pool for all heads: heads_per_pool = heads, pool_stride = 0). */
+/* Two further restrictions and one further term, for attention layers that have them (0 / NULL: none):
+ *   chunk > 0:  only j with floor(j / chunk) == floor(pos[t] / chunk) are visible (chunks counted from position 0);
+ *   bias:       float [heads, bias_len]; bias[h, min(pos[t] - j, bias_len - 1)] is added to the score (after the query's scale). */
 int qsv_latent_attention(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                          const int32_t* seq, const int32_t* pos, int window, int n_tokens, int heads, int rank,
-                         int row_width, int page, int heads_per_pool, int64_t pool_stride, int dtype, int variant, void* stream);
+                         int row_width, int page, int heads_per_pool, int64_t pool_stride, int chunk, const float* bias,
+                         int bias_len, int dtype, int variant, void* stream);
 
 int qsv_latent_attention_tile_tokens(int heads);
 int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
@@ -68,18 +93,24 @@ int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
 int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                               const int32_t* pos, const int32_t* tiles, int n_tiles, int window, int heads, int rank,
                               int row_width, int page, int key_splits, float* part_o, float* part_ml, int n_tokens,
-                              int q_first, int heads_per_pool, int64_t pool_stride, void* stream);
+                              int q_first, int heads_per_pool, int64_t pool_stride, int chunk, const float* bias, int bias_len,
+                              void* stream);
 
 /* o[t, i] *= sigmoid(g[t * g_stride + i]),  i < n. */
 int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_tokens, int n, int dtype, void* stream);
 
-/* Grouped top-k router: scores = softmax(router . h[t]) over n_experts; the experts form n_groups equal groups of neighbours,
- * a group's score is its largest score, only experts of the best keep_groups groups are eligible; the top_k eligible experts
- * with the largest scores are chosen.  idx [T, top_k] int32, weight [T, top_k] float = their scores (not renormalised).
- * bias (may be NULL, [n_experts], storage type) is added to the logits before anything else; renorm != 0 divides the chosen
- * weights by their sum (= the softmax over the chosen logits only). */
+/* Grouped top-k router: scores s = softmax(router . h[t]) over n_experts (score_fn QSV_SCORE_SOFTMAX) or sigmoid(router . h[t])
+ * (QSV_SCORE_SIGMOID); the choice goes by c = s + correction (float [n_experts], may be NULL: c = s).  The experts form n_groups
+ * equal groups of neighbours, a group's score is its largest c (group_top 1) or the sum of its two largest (group_top 2), only
+ * experts of the best keep_groups groups are eligible (the others cannot be chosen whatever their c); the top_k eligible experts
+ * with the largest c are chosen.  idx [T, top_k] int32, weight [T, top_k] float = their s times `scale`; renorm != 0 divides the
+ * chosen s by their sum first (with softmax scores: the softmax over the chosen logits only).
+ * bias (may be NULL, [n_experts], storage type) is added to the logits before anything else. */
+#define QSV_SCORE_SOFTMAX 0
+#define QSV_SCORE_SIGMOID 1
 int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, const void* bias, int renorm, int n_tokens,
-                  int width, int n_experts, int top_k, int n_groups, int keep_groups, int dtype, void* stream);
+                  int width, int n_experts, int top_k, int n_groups, int keep_groups, int score_fn, const float* correction,
+                  int group_top, float scale, int dtype, void* stream);
 
 /* Activations of the first expert product: QSV_ACT_RELU_SQ relu(z)^2; QSV_ACT_GLU: the weight rows come in pairs (2f = gate,
  * 2f + 1 = up), output f = silu(gate) * up, and the output is half as wide as the product. */
@@ -137,8 +168,10 @@ int qsv_dyt_sum_rows(void* out, const float* x, const int32_t* rows, const void*
 /* out[t] = (rms_norm(a[t]) * wa + rms_norm(b[t]) * wb) / 2 over `width`. */
 int qsv_rms_pair_mean(void* out, const void* a, const void* wa, const void* b, const void* wb, float eps, int n_tokens,
                       int width, int dtype, void* stream);
-/* out[r, f] = silu(a[r, 2f]) * a[r, 2f + 1]     a: [n_rows, 2 ff] */
-int qsv_glu(void* out, const void* a, int n_rows, int ff, int dtype, void* stream);
+/* out[r, f] = act(a[r, 2f]) * a[r, 2f + 1]     a: [n_rows, 2 ff]; act QSV_GLU_SILU or QSV_GLU_GELU_TANH (gelu in its tanh form) */
+#define QSV_GLU_SILU 0
+#define QSV_GLU_GELU_TANH 1
+int qsv_glu(void* out, const void* a, int n_rows, int ff, int act, int dtype, void* stream);
 
 /* ---- matrix-state recurrences and the attention beside them (serve_recurrent.hip) ------------------------------------------- */
 /* out[t, c] (float, [T, heads * dim]) = a_log ? exp(-exp(a_log[c / dim]) * softplus(z[t, c] + bias[c]))
@@ -159,13 +192,25 @@ int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, in
  * q, k: [T, qk_heads, dim] (head h reads h / (heads / qk_heads)), v: [T, heads, vdim], each with its row stride, of type
  * qkv_dtype; o: float [T, heads, vdim].  max_run: the longest run's tokens as the host knows them (1: every run is one decoded
  * token - a kernel without staging is used; any larger value, or 0 for unknown: the general kernel). */
+/* Variants (0 / NULL: as above): head_decay != 0: decay is float [T, heads], one factor for all rows of a head's state;
+ * kscale (float [T, heads]): k is multiplied by kscale[t, head] where it enters the state; v_cols < vdim: v has v_cols columns per
+ * head and the state's column v_cols is fed with ones (it then holds sum of decayed kscale k: a normaliser, read out by q like
+ * the others), further columns with zeros. */
 int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                        int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
                        int beta_dtype, float* state, const int32_t* runs, int n_runs, int max_run, int heads, int qk_heads,
-                       int dim, int vdim, float q_scale, void* stream);
-/* out[t, h] = o[t, h] / rms(o[t, h]) * w * gate_fn(gate[t, h]) over vdim; gate_kind 0: silu, 1: sigmoid. */
+                       int dim, int vdim, float q_scale, const float* kscale, int head_decay, int v_cols, void* stream);
+/* out[t, h] = o[t, h] / rms(o[t, h]) * w * gate_fn(gate[t, h]) over vdim; gate_kind 0: silu, 1: sigmoid.  o's heads are o_stride
+ * floats apart (0: vdim); w is [vdim], shared by the heads, or with w_per_head [heads, vdim].  den_m (float [T, heads], may be
+ * NULL): o[t, h] is first divided by max(|o[t, h, vdim]|, exp(-den_m[t, h])) + 1e-6 (o_stride > vdim: the extra column). */
 int qsv_head_rms_gate(void* out, const float* o, const void* w, const void* gate, int64_t gate_stride, int gate_kind, float eps,
-                      int n_tokens, int heads, int vdim, int dtype, void* stream);
+                      int n_tokens, int heads, int vdim, int o_stride, int w_per_head, const float* den_m, int dtype, void* stream);
+/* Exponential input and forget gates with a running maximum, per run (slot, first token, tokens, first position) and head:
+ *   li = cap tanh((zi[t, h] + bias_i[h]) / cap),  lf = logsigmoid(cap tanh((zf[t, h] + bias_f[h]) / cap)),
+ *   m_t = max(lf + m_(t-1), li),  a[t, h] = exp(lf + m_(t-1) - m_t),  b[t, h] = exp(li - m_t),  m[t, h] = m_t      (float [T, heads])
+ * m_(t-1) of a run's first token is m_state[slot, h] (0 if the run starts at position 0); the run's last m goes back there. */
+int qsv_max_gates(float* a, float* b, float* m, const void* zi, const void* zf, int64_t z_stride, const float* bias_i,
+                  const float* bias_f, float cap, float* m_state, const int32_t* runs, int n_runs, int heads, int dtype, void* stream);
 /* Rotations in the halves layout (pair p of n rotated dimensions = p and p + n / 2; rope: float [positions, 2, n / 2]):
  *   qf[t, h]           = [ 0 (vdim) | rot_k(q[t, h]) * scale ]            float [T, heads, vdim + dim]
  *   pool[g, slot[t]]   = [ rot_v(v[t, g]) | rot_k(k[t, g]) ]              [kv_heads, pool_rows, vdim + dim]

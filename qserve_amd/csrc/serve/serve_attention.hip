@@ -17,7 +17,7 @@ template <typename T, int EPL>
 __global__ __launch_bounds__(64 * NW) void latent_attention_wave_kernel(
     T* __restrict__ out, const float* __restrict__ qf, const T* pool, const int32_t* __restrict__ block_table,
     int table_stride, const int32_t* __restrict__ seq, const int32_t* __restrict__ pos, int window, int H, int rank, int R,
-    int page, int per, int64_t pool_stride) {
+    int page, int per, int64_t pool_stride, int chunk, const float* __restrict__ bias, int bias_len) {
     __shared__ float s_m[NW], s_l[NW];
     __shared__ float s_acc[NW][64 * EPL];
     const size_t t = blockIdx.x / H;
@@ -25,7 +25,9 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_wave_kernel(
     pool += (size_t)(h / per) * (size_t)pool_stride;             // heads [g per, (g + 1) per) read pool g
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const int p = pos[t];
-    const int lo = window > 0 ? max(0, p - window + 1) : 0;
+    int lo = window > 0 ? max(0, p - window + 1) : 0;
+    if (chunk > 0) lo = max(lo, p - p % chunk);                  // chunks are counted from position 0 of the sequence
+    const float* brow = bias ? bias + (size_t)h * bias_len : nullptr;
     const int32_t* bt = block_table + (size_t)seq[t] * table_stride;
     const float* qrow = qf + (t * H + h) * (size_t)R;
     float q[EPL], acc[EPL];
@@ -52,6 +54,7 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_wave_kernel(
                 d += q[i] * c[k][i];
             }
             d = wave_sum(d);
+            if (brow) d += brow[min(p - jj, bias_len - 1)];
             s[k] = ok ? d : -INFINITY;
         }
         float mx = m;
@@ -102,11 +105,12 @@ __global__ __launch_bounds__(64 * NW) void latent_attention_wave_kernel(
 
 template <typename T>
 int launch_wave(void* out, const float* qf, const void* pool, const int32_t* bt, int ts, const int32_t* seq, const int32_t* pos,
-                int window, int n, int H, int rank, int R, int page, int per, int64_t pool_stride, hipStream_t st_) {
+                int window, int n, int H, int rank, int R, int page, int per, int64_t pool_stride, int chunk, const float* bias,
+                int bias_len, hipStream_t st_) {
     const dim3 grid(n * H), block(64 * NW);
 #define QSV_ATT(E)                                                                                                        \
     hipLaunchKernelGGL((latent_attention_wave_kernel<T, E>), grid, block, 0, st_, (T*)out, qf, (const T*)pool, bt, ts, seq, pos, \
-                       window, H, rank, R, page, per, pool_stride)
+                       window, H, rank, R, page, per, pool_stride, chunk, bias, bias_len)
     if (R <= 64) QSV_ATT(1);
     else if (R <= 128) QSV_ATT(2);
     else if (R <= 192) QSV_ATT(3);
@@ -125,8 +129,10 @@ int launch_wave(void* out, const float* qf, const void* pool, const int32_t* bt,
 
 extern "C" int qsv_latent_attention(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                                     const int32_t* seq, const int32_t* pos, int window, int n, int H, int rank, int R, int page,
-                                    int heads_per_pool, int64_t pool_stride, int dtype, int variant, void* stream) {
+                                    int heads_per_pool, int64_t pool_stride, int chunk, const float* bias, int bias_len, int dtype,
+                                    int variant, void* stream) {
     QSV_REQUIRE(out && qf && pool && block_table && seq && pos, "qsv_latent_attention: null argument");
+    QSV_REQUIRE(chunk >= 0 && (!bias || bias_len > 0), "qsv_latent_attention: chunk %d, bias table of %d distances", chunk, bias_len);
     QSV_REQUIRE(n >= 0 && H > 0 && rank > 0 && R >= rank && page > 0 && table_stride > 0 && window >= 0,
                 "qsv_latent_attention: bad sizes");
     QSV_REQUIRE(heads_per_pool > 0 && H % heads_per_pool == 0 && pool_stride >= 0, "qsv_latent_attention: %d heads over pools of %d",
@@ -137,7 +143,7 @@ extern "C" int qsv_latent_attention(void* out, const float* qf, const void* pool
     int rc = QSV_OK;
     QSV_DISPATCH(dtype, "qsv_latent_attention",
                  rc = launch_wave<T>(out, qf, pool, block_table, table_stride, seq, pos, window, n, H, rank, R, page, heads_per_pool,
-                                     pool_stride, (hipStream_t)stream));
+                                     pool_stride, chunk, bias, bias_len, (hipStream_t)stream));
     if (rc != QSV_OK) return rc;
     return qsv_launch_status("qsv_latent_attention");
 }

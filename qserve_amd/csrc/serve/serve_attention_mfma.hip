@@ -31,7 +31,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     bf16_t* __restrict__ out, const float* __restrict__ qf, const bf16_t* __restrict__ pool_base,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ pos, const int32_t* __restrict__ tiles,
     int window, int H, int rank, int R, int page, int HP, int TQ, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int n_tokens, int s_lo, int s_hi, int per, int64_t pool_stride) {
+    int n_tokens, int s_lo, int s_hi, int per, int64_t pool_stride, int chunk, const float* __restrict__ bias, int bias_len) {
     constexpr int RS = 32 * RT + 8;                      // row stride (elements) of the row-major tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* Ks = (bf16_t*)smem;                          // [BN][RS]
@@ -57,15 +57,20 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     const bool row_ok = active && tok_in < ntok && head < h_end;
     const int t = t0 + (tok_in < ntok ? tok_in : 0);
     const int p_row = pos[t];
-    const int lo_row = window > 0 ? max(0, p_row - window + 1) : 0;
+    int lo_row = window > 0 ? max(0, p_row - window + 1) : 0;
+    if (chunk > 0) lo_row = max(lo_row, p_row - p_row % chunk);   // chunks are counted from position 0 of the sequence
+    const float* brow = bias ? bias + (size_t)(row_ok ? head : 0) * bias_len : nullptr;
 
     // block key range (tokens of a tile are consecutive positions; read both ends)
     const int p_first = pos[t0], p_last = pos[t0 + ntok - 1];
-    const int kstart = ((window > 0 ? max(0, p_first - window + 1) : 0) / BN) * BN;
+    int lo_first = window > 0 ? max(0, p_first - window + 1) : 0;
+    if (chunk > 0) lo_first = max(lo_first, p_first - p_first % chunk);   // (the first token's bound is the tile's lowest)
+    const int kstart = (lo_first / BN) * BN;
     // wave key range: rows of this wave's group
     const int gt_first = min(grp * TQ, ntok - 1), gt_last = min(grp * TQ + TQ - 1, ntok - 1);
     const int wp_last = p_first + gt_last;
-    const int wlo = window > 0 ? max(0, p_first + gt_first - window + 1) : 0;
+    int wlo = window > 0 ? max(0, p_first + gt_first - window + 1) : 0;
+    if (chunk > 0) wlo = max(wlo, (p_first + gt_first) - (p_first + gt_first) % chunk);
 
     // Q fragments (B operand of S^T): the 8 consecutive elements 32 s + 8 g4 of this lane's row
     v4u qfrag[RT];
@@ -149,6 +154,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
             for (int r = 0; r < 4; ++r) {
                 const int key = k0 + 16 * mt + 4 * g4 + r;
                 const bool vis = key <= p_row && key >= lo_row;
+                if (brow && vis) sacc[mt][r] += brow[min(p_row - key, bias_len - 1)];
                 sacc[mt][r] = vis ? sacc[mt][r] : -INFINITY;
                 tmax = fmaxf(tmax, sacc[mt][r]);
             }
@@ -304,7 +310,9 @@ extern "C" int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype) 
 extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, const int32_t* block_table,
                                          int table_stride, const int32_t* pos, const int32_t* tiles, int n_tiles, int window,
                                          int H, int rank, int R, int page, int key_splits, float* part_o, float* part_ml,
-                                         int n_tokens, int q_first, int heads_per_pool, int64_t pool_stride, void* stream) {
+                                         int n_tokens, int q_first, int heads_per_pool, int64_t pool_stride, int chunk,
+                                         const float* bias, int bias_len, void* stream) {
+    QSV_REQUIRE(chunk >= 0 && (!bias || bias_len > 0), "qsv_latent_attention_mfma: chunk %d, bias table of %d distances", chunk, bias_len);
     QSV_REQUIRE(out && qf && pool && block_table && pos && tiles, "qsv_latent_attention_mfma: null argument");
     QSV_REQUIRE(qsv_latent_attention_mfma_ok(rank, R, QSV_BF16) && R >= rank && H > 0 && page > 0 && page % BN == 0 && window >= 0 && n_tiles >= 0,
                 "qsv_latent_attention_mfma: sizes not supported (rank %d, row %d)", rank, R);
@@ -330,7 +338,7 @@ extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void*
         }                                                                                                                    \
         hipLaunchKernelGGL((latent_attention_mfma_kernel<RT, CT>), grid, block, lds, (hipStream_t)stream, (bf16_t*)out, qf,  \
                            (const bf16_t*)pool, block_table, table_stride, pos, tiles, window, H, rank, R, page, g.HP, g.TQ, \
-                           part_o, part_ml, n_tokens, s_lo, s_hi, heads_per_pool, pool_stride);                              \
+                           part_o, part_ml, n_tokens, s_lo, s_hi, heads_per_pool, pool_stride, chunk, bias, bias_len);        \
     } while (0)
     if (rt <= 4 && ct <= 8) QSV_MFMA(4, 8);
     else if (rt <= 6 && ct <= 12) QSV_MFMA(6, 12);

@@ -35,17 +35,22 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
     }
 }
 
-// One workgroup per token.  z = router . h by the four waves (16-byte loads where the width allows), then wave 0 selects:
-// softmax, group maxima, the best groups and the top experts by repeated wave-wide argmax.  Ties go to the lower index, for
-// groups and for experts.
+// One workgroup per token.  z = router . h by the four waves (16-byte loads where the width allows), then wave 0 selects by
+// repeated wave-wide argmax.  Scores s = softmax(z) over all experts (score_fn 0) or sigmoid(z) (1); the CHOICE goes by c = s +
+// correction (correction may be NULL), the WEIGHTS are the chosen experts' s times `scale` (divided by their sum first if renorm).
+// A group's score is its largest c (group_top 1) or the sum of its two largest (2); experts outside the `keep` best groups cannot
+// be chosen, however low the others' c.  Ties go to the lower index, for groups and for experts.
 template <typename T>
 __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx, float* __restrict__ weight,
                                                        const T* __restrict__ h, const T* __restrict__ router,
                                                        const T* __restrict__ bias, int renorm, int D, int E, int top_k, int G,
-                                                       int keep) {
+                                                       int keep, int score_fn, const float* __restrict__ correction,
+                                                       int group_top, float scale) {
     __shared__ float s[MAX_EXPERTS];
+    __shared__ float c[MAX_EXPERTS];
     __shared__ float gs[MAX_EXPERTS];
     __shared__ unsigned char ok[MAX_EXPERTS];
+    __shared__ unsigned char gtaken[MAX_EXPERTS];
     const size_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     const T* x = h + t * D;
@@ -53,10 +58,10 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
         const T* r = router + (size_t)e * D;
         float d = 0.f;
         if (D % 8 == 0) {
-            for (int c = lane * 8; c < D; c += 64 * 8) {
+            for (int cc = lane * 8; cc < D; cc += 64 * 8) {
                 float a[8], b[8];
-                load8(r + c, a);
-                load8(x + c, b);
+                load8(r + cc, a);
+                load8(x + cc, b);
 #pragma unroll
                 for (int q = 0; q < 8; ++q) d += a[q] * b[q];
             }
@@ -69,30 +74,43 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
     __syncthreads();
     // (the other three waves only keep the barriers company from here on: the selection is a few hundred steps of one wave)
     const bool sel = w == 0;
-    float inv = 0.f;
-    if (sel) {                                              // softmax over all experts
-        float mx = -INFINITY;
-        for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
-        mx = wave_max(mx);
-        float sum = 0.f;
-        for (int e = lane; e < E; e += 64) {
-            const float p = expf(s[e] - mx);
-            s[e] = p;
-            sum += p;
+    if (sel) {
+        if (score_fn == 0) {                                // softmax over all experts
+            float mx = -INFINITY;
+            for (int e = lane; e < E; e += 64) mx = fmaxf(mx, s[e]);
+            mx = wave_max(mx);
+            float sum = 0.f;
+            for (int e = lane; e < E; e += 64) {
+                const float p = expf(s[e] - mx);
+                s[e] = p;
+                sum += p;
+            }
+            const float inv = 1.0f / wave_sum(sum);
+            for (int e = lane; e < E; e += 64) s[e] *= inv;
+        } else {
+            for (int e = lane; e < E; e += 64) s[e] = 1.0f / (1.0f + expf(-s[e]));
         }
-        inv = 1.0f / wave_sum(sum);
         for (int e = lane; e < E; e += 64) {
-            s[e] *= inv;
+            c[e] = correction ? s[e] + correction[e] : s[e];
             ok[e] = 0;
         }
     }
     __syncthreads();
     const int per = E / G;
-    if (sel) {                                              // group maxima
+    if (sel) {                                              // group scores
         for (int g = lane; g < G; g += 64) {
-            float v = s[g * per];
-            for (int e = 1; e < per; ++e) v = fmaxf(v, s[g * per + e]);
-            gs[g] = v;
+            float v1 = c[g * per], v2 = -INFINITY;          // the two largest
+            for (int e = 1; e < per; ++e) {
+                const float v = c[g * per + e];
+                if (v > v1) {
+                    v2 = v1;
+                    v1 = v;
+                } else if (v > v2) {
+                    v2 = v;
+                }
+            }
+            gs[g] = (group_top == 2 && per > 1) ? v1 + v2 : v1;
+            gtaken[g] = 0;
         }
     }
     __syncthreads();
@@ -101,12 +119,12 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
             float bv = 0.f;
             int bi = -1;
             for (int g = lane; g < G; g += 64)
-                if (gs[g] >= 0.f && (bi < 0 || gs[g] > bv)) {
+                if (!gtaken[g] && (bi < 0 || gs[g] > bv)) {
                     bv = gs[g];
                     bi = g;
                 }
             wave_argmax(bv, bi);
-            if (lane == 0) gs[bi] = -1.f;                   // scores are probabilities: -1 marks a taken group
+            if (lane == 0) gtaken[bi] = 1;
             for (int e = lane; e < per; e += 64) ok[bi * per + e] = 1;
         }
         __syncthreads();
@@ -117,23 +135,27 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
             float bv = 0.f;
             int bi = -1;
             for (int e = lane; e < E; e += 64)
-                if (ok[e] && (bi < 0 || s[e] > bv)) {
-                    bv = s[e];
+                if (ok[e] && (bi < 0 || c[e] > bv)) {
+                    bv = c[e];
                     bi = e;
                 }
             wave_argmax(bv, bi);
             if (lane == 0) {
                 ok[bi] = 0;
                 idx[t * top_k + k] = bi;
-                weight[t * top_k + k] = bv;
-                chosen += bv;
+                weight[t * top_k + k] = s[bi];
+                chosen += s[bi];
             }
         }
         __syncthreads();
     }
     // weights over the chosen only: p_i / sum of the chosen p = the softmax over the chosen logits
-    if (renorm && sel && lane == 0)
-        for (int k = 0; k < top_k; ++k) weight[t * top_k + k] /= chosen;
+    if (sel && lane == 0 && (renorm || scale != 1.0f))
+        for (int k = 0; k < top_k; ++k) {
+            float v = weight[t * top_k + k];
+            if (renorm) v /= chosen;
+            weight[t * top_k + k] = v * scale;
+        }
 }
 
 // Activation of the first expert product.  ACT_GLU: the weight rows come in pairs (2f = gate, 2f + 1 = up) and output f is
@@ -445,7 +467,10 @@ extern "C" int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, cons
 }
 
 extern "C" int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router, const void* bias, int renorm, int n,
-                             int D, int E, int top_k, int G, int keep, int dtype, void* stream) {
+                             int D, int E, int top_k, int G, int keep, int score_fn, const float* correction, int group_top,
+                             float scale, int dtype, void* stream) {
+    QSV_REQUIRE((score_fn == 0 || score_fn == 1) && (group_top == 1 || group_top == 2), "qsv_moe_route: score function %d, group score %d",
+                score_fn, group_top);
     QSV_REQUIRE(idx && weight && h && router && n >= 0 && D > 0, "qsv_moe_route: bad arguments");
     QSV_REQUIRE(E > 0 && E <= MAX_EXPERTS && G > 0 && E % G == 0 && keep > 0 && keep <= G && top_k > 0 &&
                     top_k <= keep * (E / G),
@@ -453,7 +478,8 @@ extern "C" int qsv_moe_route(int32_t* idx, float* weight, const void* h, const v
     if (n == 0) return QSV_OK;
     QSV_DISPATCH(dtype, "qsv_moe_route",
                  hipLaunchKernelGGL(moe_route_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, idx, weight, (const T*)h,
-                                    (const T*)router, (const T*)bias, renorm, D, E, top_k, G, keep));
+                                    (const T*)router, (const T*)bias, renorm, D, E, top_k, G, keep, score_fn, correction,
+                                    group_top, scale));
     return qsv_launch_status("qsv_moe_route");
 }
 

@@ -111,7 +111,8 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__
                                                              int64_t v_stride, const float* __restrict__ decay,
                                                              const TB* __restrict__ beta, int64_t beta_stride,
                                                              float* __restrict__ state, const int32_t* __restrict__ runs, int H,
-                                                             int QH, int dim, int vdim, int lpc_log, int CT, float q_scale) {
+                                                             int QH, int dim, int vdim, int lpc_log, int CT, float q_scale,
+                                                             const float* __restrict__ kscale, int head_decay, int v_cols) {
     static_assert(R == 4 || R == 8 || R == 16, "rows per lane");
     extern __shared__ __attribute__((aligned(16))) float sm[];
     const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nthr >> 6;
@@ -144,10 +145,20 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__
                 if (idx < nk) {
                     const int seg = idx >> dimp_log, r = idx & (DIMP - 1), tt = seg / 3, which = seg - 3 * tt;
                     const size_t t = (size_t)(first + c0 + tt);
-                    if (r < dim)
-                        val = which == 0 ? ld4(k, t * k_stride + (size_t)qh * dim + r)
-                            : which == 1 ? ld4(q, t * q_stride + (size_t)qh * dim + r)
-                                         : ld4(decay, (t * H + h) * (size_t)dim + r);
+                    if (r < dim) {
+                        if (which == 2 && head_decay) {
+                            const float g = decay[t * H + h];
+                            val = make_float4(g, g, g, g);
+                        } else {
+                            val = which == 0 ? ld4(k, t * k_stride + (size_t)qh * dim + r)
+                                : which == 1 ? ld4(q, t * q_stride + (size_t)qh * dim + r)
+                                             : ld4(decay, (t * H + h) * (size_t)dim + r);
+                            if (which == 0 && kscale) {
+                                const float b = kscale[t * H + h];
+                                val.x *= b; val.y *= b; val.z *= b; val.w *= b;
+                            }
+                        }
+                    }
                 }
                 pk[4 * i] = val.x; pk[4 * i + 1] = val.y; pk[4 * i + 2] = val.z; pk[4 * i + 3] = val.w;
             }
@@ -157,7 +168,8 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__
                 float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (idx < nv) {
                     const int tt = idx >> vb_log, c = idx & (VB - 1), jj = blockIdx.z * VB + c;
-                    if (jj < vdim) val = ld4(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * vdim + jj);
+                    if (jj < v_cols) val = ld4(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * v_cols + jj);
+                    else if (jj == v_cols && jj < vdim) val.x = 1.0f;        // the state's column of ones (a state wider than v)
                 }
                 pv[4 * i] = val.x; pv[4 * i + 1] = val.y; pv[4 * i + 2] = val.z; pv[4 * i + 3] = val.w;
             }
@@ -170,9 +182,9 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__
                     const int seg = idx >> dimp_log, r = idx & (DIMP - 1), tt = seg / 3, which = seg - 3 * tt;
                     const size_t t = (size_t)(first + c0 + tt);
                     if (r < dim)
-                        val = which == 0 ? ld(k, t * k_stride + (size_t)qh * dim + r)
+                        val = which == 0 ? ld(k, t * k_stride + (size_t)qh * dim + r) * (kscale ? kscale[t * H + h] : 1.0f)
                             : which == 1 ? ld(q, t * q_stride + (size_t)qh * dim + r)
-                                         : decay[(t * H + h) * (size_t)dim + r];
+                                         : (head_decay ? decay[t * H + h] : decay[(t * H + h) * (size_t)dim + r]);
                 }
                 pk[i] = val;
             }
@@ -182,7 +194,8 @@ __global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__
                 float val = 0.f;
                 if (idx < nv) {
                     const int tt = idx >> vb_log, c = idx & (VB - 1), jj = blockIdx.z * VB + c;
-                    if (jj < vdim) val = ld(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * vdim + jj);
+                    if (jj < v_cols) val = ld(v, (size_t)(first + c0 + tt) * v_stride + (size_t)h * v_cols + jj);
+                    else if (jj == v_cols && jj < vdim) val = 1.0f;
                 }
                 pv[i] = val;
             }
@@ -313,7 +326,8 @@ __global__ __launch_bounds__(256) void recurrent_step_kernel(float* __restrict__
                                                              int64_t v_stride, const float* __restrict__ decay,
                                                              const TB* __restrict__ beta, int64_t beta_stride,
                                                              float* __restrict__ state, const int32_t* __restrict__ runs, int H,
-                                                             int QH, int dim, int vdim, int lpc_log, float q_scale) {
+                                                             int QH, int dim, int vdim, int lpc_log, float q_scale,
+                                                             const float* __restrict__ kscale, int head_decay, int v_cols) {
     constexpr int R = 8;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lpc = 1 << lpc_log, cols = 64 >> lpc_log;
@@ -326,15 +340,16 @@ __global__ __launch_bounds__(256) void recurrent_step_kernel(float* __restrict__
     const int h = blockIdx.y, qh = h / (H / QH);
     float* Sg = state + (((size_t)slot * H + h) * dim) * (size_t)vdim + (col_ok ? j : 0);
     float S[R], kc[R], qc[R], gc[R];
+    const float kb = kscale ? kscale[t * H + h] : 1.0f;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
         const bool ok = r0 + i < dim;
         S[i] = (!fresh && col_ok && ok) ? Sg[(size_t)(r0 + i) * vdim] : 0.f;
-        kc[i] = ok ? ld(k, t * k_stride + (size_t)qh * dim + r0 + i) : 0.f;
+        kc[i] = ok ? ld(k, t * k_stride + (size_t)qh * dim + r0 + i) * kb : 0.f;
         qc[i] = ok ? ld(q, t * q_stride + (size_t)qh * dim + r0 + i) : 0.f;
-        gc[i] = ok ? decay[(t * H + h) * (size_t)dim + r0 + i] : 0.f;
+        gc[i] = ok ? (head_decay ? decay[t * H + h] : decay[(t * H + h) * (size_t)dim + r0 + i]) : 0.f;
     }
-    const float vc = col_ok ? ld(v, t * v_stride + (size_t)h * vdim + j) : 0.f;
+    const float vc = !col_ok ? 0.f : j < v_cols ? ld(v, t * v_stride + (size_t)h * v_cols + j) : j == v_cols ? 1.0f : 0.f;
     float acc = 0.f;
     if (DELTA) {
 #pragma unroll
@@ -364,25 +379,72 @@ __global__ __launch_bounds__(256) void recurrent_step_kernel(float* __restrict__
         if (r0 + i < dim) Sg[(size_t)(r0 + i) * vdim] = S[i];
 }
 
-// ---- per-head RMS norm of the read-out, times a weight shared by the heads, times a gate ---------------------------------------
-// gate_kind 0: silu(g), 1: sigmoid(g)
+// ---- per-head RMS norm of the read-out, times a weight, times a gate ------------------------------------------------------------
+// gate_kind 0: silu(g), 1: sigmoid(g).  o rows are o_stride floats apart per head (>= vdim); w_stride 0: one weight row shared by
+// the heads, vdim: a row per head.  den_m != NULL: before the norm the read-out is divided by max(|o[vdim]|, exp(-den_m[t, h])) +
+// 1e-6, o[vdim] being the head's extra column (the normaliser's dot product with the query).
 template <typename T>
 __global__ __launch_bounds__(NT) void head_rms_gate_kernel(T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ w,
                                                            const T* __restrict__ gate, int64_t gate_stride, int gate_kind, float eps,
-                                                           int H, int vdim) {
+                                                           int H, int vdim, int o_stride, int w_stride,
+                                                           const float* __restrict__ den_m) {
     const size_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     for (int h = wv; h < H; h += NW) {
-        const float* oh = o + (t * H + h) * (size_t)vdim;
+        const float* oh = o + (t * H + h) * (size_t)o_stride;
+        const float sc = den_m ? 1.0f / (fmaxf(fabsf(oh[vdim]), expf(-den_m[t * H + h])) + 1e-6f) : 1.0f;
         float s = 0.f;
-        for (int e = lane; e < vdim; e += 64) s += oh[e] * oh[e];
+        for (int e = lane; e < vdim; e += 64) s += (oh[e] * sc) * (oh[e] * sc);
         const float inv = 1.0f / sqrtf(wave_sum(s) / (float)vdim + eps);
         for (int e = lane; e < vdim; e += 64) {
             const float g = ld(gate, t * gate_stride + (size_t)h * vdim + e);
             const float sg = 1.0f / (1.0f + expf(-g));
-            st(out, (t * H + h) * (size_t)vdim + e, oh[e] * inv * ld(w, e) * (gate_kind == 0 ? g * sg : sg));
+            st(out, (t * H + h) * (size_t)vdim + e, oh[e] * sc * inv * ld(w, (size_t)h * w_stride + e) * (gate_kind == 0 ? g * sg : sg));
         }
     }
+}
+
+// ---- exponential gates kept in range by a running maximum (mLSTM) ----------------------------------------------------------------
+// Per (run, head) one wave; a lane takes one token of 64 at a time.  li = cap tanh((z_i + b_i) / cap), lf = logsigmoid(cap tanh((z_f
+// + b_f) / cap)); m_t = max(lf_t + m_(t-1), li_t) is a scan over the maps x -> max(x + A, B), which compose to (A1 + A2, max(B1 + A2,
+// B2)); decay a_t = exp(lf_t + m_(t-1) - m_t), input scale b_t = exp(li_t - m_t).  m of a run's last token goes back to the state
+// (a run that starts its sequence starts from m = 0).
+__device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+template <typename T>
+__global__ __launch_bounds__(64) void max_gates_kernel(float* __restrict__ a_out, float* __restrict__ b_out, float* __restrict__ m_out,
+                                                       const T* __restrict__ zi, const T* __restrict__ zf, int64_t z_stride,
+                                                       const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap,
+                                                       float* __restrict__ m_state, const int32_t* __restrict__ runs, int H) {
+    const int lane = threadIdx.x;
+    const int slot = runs[4 * blockIdx.x], first = runs[4 * blockIdx.x + 1], n = runs[4 * blockIdx.x + 2];
+    const int h = blockIdx.y;
+    float carry = runs[4 * blockIdx.x + 3] == 0 ? 0.f : m_state[(size_t)slot * H + h];
+    const float inv_cap = 1.0f / cap;
+    for (int c0 = 0; c0 < n; c0 += 64) {
+        const bool ok = c0 + lane < n;
+        const size_t t = (size_t)first + c0 + (ok ? lane : 0);
+        const float li = cap * tanhf((ld(zi, t * z_stride + h) + bias_i[h]) * inv_cap);
+        const float lf = log_sigmoid(cap * tanhf((ld(zf, t * z_stride + h) + bias_f[h]) * inv_cap));
+        float A = ok ? lf : 0.f, B = ok ? li : -INFINITY;       // (a lane past the end is the identity map)
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const float pA = __shfl_up(A, o, 64), pB = __shfl_up(B, o, 64);
+            if (lane >= o) {
+                B = fmaxf(pB + A, B);
+                A = pA + A;
+            }
+        }
+        const float m = fmaxf(carry + A, B);
+        float prev = __shfl_up(m, 1, 64);
+        if (lane == 0) prev = carry;
+        if (ok) {
+            a_out[t * H + h] = expf(lf + prev - m);
+            b_out[t * H + h] = expf(li - m);
+            m_out[t * H + h] = m;
+        }
+        carry = __shfl(m, min(63, n - c0 - 1), 64);
+    }
+    if (lane == 0) m_state[(size_t)slot * H + h] = carry;
 }
 
 // ---- rotations, halves layout: pair p of n rotated dimensions = (p, p + n / 2); rope [positions, 2, n / 2] -------------------
@@ -468,8 +530,10 @@ extern "C" int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, 
 extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                                   int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
                                   int beta_dtype, float* state, const int32_t* runs, int n_runs, int max_run, int heads, int qk_heads,
-                                  int dim, int vdim, float q_scale, void* stream) {
+                                  int dim, int vdim, float q_scale, const float* kscale, int head_decay, int v_cols, void* stream) {
     QSV_REQUIRE(o && q && k && v && decay && state && runs, "qsv_recurrent_scan: null argument");
+    if (v_cols <= 0) v_cols = vdim;
+    QSV_REQUIRE(v_cols <= vdim, "qsv_recurrent_scan: %d value columns for a state of %d", v_cols, vdim);
     if (max_run == 1 && n_runs > 0 && dim <= 64 * 8 && heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && vdim > 0 && heads <= 65535) {
         int lpc = 1, lpc_log = 0;
         while (lpc * 8 < dim) lpc <<= 1, ++lpc_log;
@@ -479,7 +543,7 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
 #define QSV_STEP(TQ, TB, DELTA)                                                                                              \
     hipLaunchKernelGGL((recurrent_step_kernel<TQ, TB, DELTA>), grid, block, 0, (hipStream_t)stream, o, (const TQ*)q, q_stride,    \
                        (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta, beta_stride, state, runs, heads,  \
-                       qk_heads, dim, vdim, lpc_log, q_scale)
+                       qk_heads, dim, vdim, lpc_log, q_scale, kscale, head_decay, v_cols)
         if (beta) {
             if (qkv_dtype == QSV_F32 && beta_dtype == QSV_F32) QSV_STEP(float, float, true);
             else if (qkv_dtype == QSV_F32 && beta_dtype == QSV_BF16) QSV_STEP(float, bf16_t, true);
@@ -525,13 +589,13 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     const dim3 grid(n_runs, heads, (vdim + VB - 1) / VB), block(nthr);
     QSV_REQUIRE(grid.z <= 65535, "qsv_recurrent_scan: too many column blocks");
     const size_t el = qkv_dtype == QSV_F32 ? 4 : 2;
-    const bool vec = dim % 4 == 0 && vdim % 4 == 0 && VB % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 &&
+    const bool vec = dim % 4 == 0 && vdim % 4 == 0 && v_cols % 4 == 0 && VB % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 &&
                      (uintptr_t)q % (4 * el) == 0 && (uintptr_t)k % (4 * el) == 0 && (uintptr_t)v % (4 * el) == 0 &&
                      (uintptr_t)decay % 16 == 0;
 #define QSV_SCAN_V(TQ, TB, DELTA, VEC, RR, CC)                                                                               \
     hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, VEC, RR, CC>), grid, block, lds, (hipStream_t)stream, o,            \
                        (const TQ*)q, q_stride, (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta,         \
-                       beta_stride, state, runs, heads, qk_heads, dim, vdim, lpc_log, CT, q_scale)
+                       beta_stride, state, runs, heads, qk_heads, dim, vdim, lpc_log, CT, q_scale, kscale, head_decay, v_cols)
 #define QSV_SCAN(TQ, TB, DELTA)                                \
     do {                                                       \
         if (vec && R == 8) QSV_SCAN_V(TQ, TB, DELTA, true, 8, 1);   \
@@ -555,15 +619,31 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
 }
 
 extern "C" int qsv_head_rms_gate(void* out, const float* o, const void* w, const void* gate, int64_t gate_stride, int gate_kind,
-                                 float eps, int n_tokens, int heads, int vdim, int dtype, void* stream) {
+                                 float eps, int n_tokens, int heads, int vdim, int o_stride, int w_per_head, const float* den_m,
+                                 int dtype, void* stream) {
     QSV_REQUIRE(out && o && w && gate && n_tokens >= 0 && heads > 0 && vdim > 0 && gate_stride >= (int64_t)heads * vdim &&
                     (gate_kind == 0 || gate_kind == 1),
                 "qsv_head_rms_gate: bad arguments");
+    if (o_stride <= 0) o_stride = vdim;
+    QSV_REQUIRE(o_stride >= vdim && (!den_m || o_stride > vdim), "qsv_head_rms_gate: read-out rows of %d floats for %d values%s",
+                o_stride, vdim, den_m ? " and the normaliser's column" : "");
     if (n_tokens == 0) return QSV_OK;
     QSV_DISPATCH(dtype, "qsv_head_rms_gate",
                  hipLaunchKernelGGL(head_rms_gate_kernel<T>, dim3(n_tokens), dim3(NT), 0, (hipStream_t)stream, (T*)out, o, (const T*)w,
-                                    (const T*)gate, gate_stride, gate_kind, eps, heads, vdim));
+                                    (const T*)gate, gate_stride, gate_kind, eps, heads, vdim, o_stride, w_per_head ? vdim : 0, den_m));
     return qsv_launch_status("qsv_head_rms_gate");
+}
+
+extern "C" int qsv_max_gates(float* a, float* b, float* m, const void* zi, const void* zf, int64_t z_stride, const float* bias_i,
+                             const float* bias_f, float cap, float* m_state, const int32_t* runs, int n_runs, int heads, int dtype,
+                             void* stream) {
+    QSV_REQUIRE(a && b && m && zi && zf && bias_i && bias_f && m_state && runs, "qsv_max_gates: null argument");
+    QSV_REQUIRE(cap > 0.f && heads > 0 && heads <= 65535 && n_runs >= 0 && z_stride >= heads, "qsv_max_gates: bad sizes");
+    if (n_runs == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_max_gates",
+                 hipLaunchKernelGGL(max_gates_kernel<T>, dim3(n_runs, heads), dim3(64), 0, (hipStream_t)stream, a, b, m, (const T*)zi,
+                                    (const T*)zf, z_stride, bias_i, bias_f, cap, m_state, runs, heads));
+    return qsv_launch_status("qsv_max_gates");
 }
 
 extern "C" int qsv_attention_prep(float* qf, void* pool, int64_t pool_rows, const void* proj, int64_t stride, int q_off, int k_off,

@@ -214,3 +214,147 @@ extern "C" int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_
                                     g_stride, n));
     return qsv_launch_status("qsv_sigmoid_gate");
 }
+
+// ---- embedding with a sinusoidal position vector ---------------------------------------------------------------------------------
+// x[t, 2i] = table[tok, 2i] * scale + sin(pos * freq[i]),  x[t, 2i + 1] = ... + cos(pos * freq[i]); the angle is a float product.
+template <typename T>
+__global__ __launch_bounds__(NT) void embed_sinusoid_kernel(float* __restrict__ x, const T* __restrict__ table,
+                                                            const int32_t* __restrict__ tokens, const int32_t* __restrict__ pos,
+                                                            const float* __restrict__ freq, float scale, int D) {
+    const size_t t = blockIdx.x;
+    const T* row = table + (size_t)tokens[t] * D;
+    const float p = (float)pos[t];
+    for (int i = threadIdx.x; i < D; i += NT) {
+        const float a = p * freq[i >> 1];
+        x[t * D + i] = ld(row, i) * scale + ((i & 1) ? cosf(a) : sinf(a));
+    }
+}
+extern "C" int qsv_embed_sinusoid(float* x, const void* table, const int32_t* tokens, const int32_t* pos, const float* freq,
+                                  float scale, int n, int D, int dtype, void* stream) {
+    QSV_REQUIRE(x && table && tokens && pos && freq && n >= 0 && D > 0, "qsv_embed_sinusoid: bad arguments");
+    if (n == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_embed_sinusoid",
+                 hipLaunchKernelGGL(embed_sinusoid_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (const T*)table, tokens, pos,
+                                    freq, scale, D));
+    return qsv_launch_status("qsv_embed_sinusoid");
+}
+
+// ---- x += a + (b + c); h = rms_norm(x) * w -----------------------------------------------------------------------------------------
+// a, b, c: the sublayers' outputs (each may be NULL); h (may be NULL: no norm) is the next layer's input in the storage type.
+template <typename T>
+__global__ __launch_bounds__(NT) void add_rms_norm_kernel(float* __restrict__ x, T* __restrict__ h, const T* __restrict__ a,
+                                                          const T* __restrict__ b, const T* __restrict__ c, const T* __restrict__ w,
+                                                          float eps, int D) {
+    __shared__ float red[NT / 64 + 1];
+    const size_t t = blockIdx.x;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < D; i += NT) {
+        float v = x[t * D + i];
+        if (a || b || c) {
+            float y = 0.f;
+            if (b) y = ld(b, t * D + i);
+            if (c) y += ld(c, t * D + i);
+            if (a) y = ld(a, t * D + i) + y;
+            v += y;
+            x[t * D + i] = v;
+        }
+        s += v * v;
+    }
+    if (!h) return;
+    const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
+    for (int i = threadIdx.x; i < D; i += NT) st(h, t * D + i, x[t * D + i] * inv * ld(w, i));   // (this thread's own writes)
+}
+extern "C" int qsv_add_rms_norm(float* x, void* h, const void* a, const void* b, const void* c, const void* w, float eps, int n,
+                                int D, int dtype, void* stream) {
+    QSV_REQUIRE(x && n >= 0 && D > 0 && (!h || w), "qsv_add_rms_norm: bad arguments");
+    if (n == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_add_rms_norm",
+                 hipLaunchKernelGGL(add_rms_norm_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (T*)h, (const T*)a, (const T*)b,
+                                    (const T*)c, (const T*)w, eps, D));
+    return qsv_launch_status("qsv_add_rms_norm");
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void rms_norm_rows_kernel(T* __restrict__ out, const float* __restrict__ x,
+                                                           const int32_t* __restrict__ rows, const T* __restrict__ w, float eps,
+                                                           int D) {
+    __shared__ float red[NT / 64 + 1];
+    const size_t r = blockIdx.x;
+    const float* xr = x + (size_t)(rows ? rows[r] : (int32_t)r) * D;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < D; i += NT) s += xr[i] * xr[i];
+    const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
+    for (int i = threadIdx.x; i < D; i += NT) st(out, r * D + i, xr[i] * inv * ld(w, i));
+}
+extern "C" int qsv_rms_norm_rows(void* out, const float* x, const int32_t* rows, const void* w, float eps, int n, int D, int dtype,
+                                 void* stream) {
+    QSV_REQUIRE(out && x && w && n >= 0 && D > 0, "qsv_rms_norm_rows: bad arguments");
+    if (n == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_rms_norm_rows",
+                 hipLaunchKernelGGL(rms_norm_rows_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, (T*)out, x, rows, (const T*)w,
+                                    eps, D));
+    return qsv_launch_status("qsv_rms_norm_rows");
+}
+
+// ---- attention with queries and keys normed over all heads at once, and values blended with an earlier layer's ------------------
+//   qf[t, h]          = [ 0 (vdim) | rms_norm(q[t])[h] * q_w[h] * scale ]       float [T, heads, vdim + dim]; the norm runs over all
+//   pool[g, slot[t]]  = [ v'[t, g] | rms_norm(k[t])[g] * k_w[g] ]               heads * dim (kv_heads * dim) values of the projection
+//   v' = (1 - mix) v + mix v_first  where v_first (row stride vf_stride, [kv_heads * vdim] per token) is given, else v.
+template <typename T>
+__global__ __launch_bounds__(NT) void normed_attention_prep_kernel(float* __restrict__ qf, T* __restrict__ pool, int64_t pool_rows,
+                                                                   const T* __restrict__ proj, int64_t stride, int q_off, int k_off,
+                                                                   int v_off, int H, int G, int dim, int vdim,
+                                                                   const T* __restrict__ q_w, const T* __restrict__ k_w, float eps,
+                                                                   float scale, const T* __restrict__ v_first, int64_t vf_stride,
+                                                                   float mix, const int64_t* __restrict__ slot) {
+    __shared__ float red[NT / 64 + 1];
+    const size_t t = blockIdx.x;
+    const int R = vdim + dim;
+    const T* row = proj + t * stride;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < H * dim; i += NT) {
+        const float v = ld(row, q_off + i);
+        s += v * v;
+    }
+    const float qinv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)(H * dim) + eps);
+    s = 0.f;
+    for (int i = threadIdx.x; i < G * dim; i += NT) {
+        const float v = ld(row, k_off + i);
+        s += v * v;
+    }
+    const float kinv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)(G * dim) + eps);
+    for (int idx = threadIdx.x; idx < H * R; idx += NT) {
+        const int h = idx / R, c = idx - h * R;
+        const int e = h * dim + c - vdim;
+        qf[t * H * (size_t)R + idx] = c < vdim ? 0.f : ld(row, q_off + e) * qinv * ld(q_w, e) * scale;
+    }
+    const size_t dst = (size_t)slot[t];
+    for (int idx = threadIdx.x; idx < G * R; idx += NT) {
+        const int g = idx / R, c = idx - g * R;
+        float val;
+        if (c < vdim) {
+            val = ld(row, v_off + g * vdim + c);
+            if (v_first) val = (1.0f - mix) * val + mix * ld(v_first, t * vf_stride + g * vdim + c);
+        } else {
+            const int e = g * dim + c - vdim;
+            val = ld(row, k_off + e) * kinv * ld(k_w, e);
+        }
+        st(pool, ((size_t)g * pool_rows + dst) * R + c, val);
+    }
+}
+extern "C" int qsv_normed_attention_prep(float* qf, void* pool, int64_t pool_rows, const void* proj, int64_t stride, int q_off,
+                                         int k_off, int v_off, int heads, int kv_heads, int dim, int vdim, const void* q_w,
+                                         const void* k_w, float eps, float scale, const void* v_first, int64_t vf_stride, float mix,
+                                         const int64_t* slot, int n, int dtype, void* stream) {
+    QSV_REQUIRE(qf && pool && proj && q_w && k_w && slot, "qsv_normed_attention_prep: null argument");
+    QSV_REQUIRE(heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0 && q_off >= 0 && k_off >= 0 && v_off >= 0 &&
+                    q_off + (int64_t)heads * dim <= stride && k_off + (int64_t)kv_heads * dim <= stride &&
+                    v_off + (int64_t)kv_heads * vdim <= stride && n >= 0 && (!v_first || vf_stride >= (int64_t)kv_heads * vdim),
+                "qsv_normed_attention_prep: bad sizes");
+    if (n == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_normed_attention_prep",
+                 hipLaunchKernelGGL(normed_attention_prep_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, qf, (T*)pool, pool_rows,
+                                    (const T*)proj, stride, q_off, k_off, v_off, heads, kv_heads, dim, vdim, (const T*)q_w,
+                                    (const T*)k_w, eps, scale, (const T*)v_first, vf_stride, mix, slot));
+    return qsv_launch_status("qsv_normed_attention_prep");
+}

@@ -33,16 +33,19 @@ def _interleave(gate, up):
 
 
 class GatedFeedForward:
-    """Dense gated feed-forward: down . (silu(gate . h) * (up . h)), no biases."""
+    """Dense gated feed-forward: down . (act(gate . h) * (up . h)), no biases; act: "silu" or "gelu_tanh"."""
 
-    def __init__(self, ops, *, gate, up, down):
+    def __init__(self, ops, *, gate, up, down, act="silu"):
         if gate.shape != up.shape or down.shape != (gate.size(1), gate.size(0)):
             raise ValueError("gated feed-forward: gate / up / down shapes do not fit each other")
-        self.ops, self.w_in, self.w_down = ops, _interleave(gate, up), down.contiguous()
+        if act not in ("silu", "gelu_tanh"):
+            raise ValueError(f"gated feed-forward: unknown activation {act!r}")
+        self.ops, self.w_in, self.w_down, self.act = ops, _interleave(gate, up), down.contiguous(), act
 
     def __call__(self, h):
         from .ops import linear
-        return linear(self.ops.glu(linear(h, self.w_in)), self.w_down)
+        a = linear(h, self.w_in)
+        return linear(self.ops.glu(a) if self.act == "silu" else self.ops.glu(a, self.act), self.w_down)
 
 
 class TopKGatedMoE:
@@ -65,3 +68,32 @@ class TopKGatedMoE:
     def __call__(self, h):
         idx, wt = self.ops.moe_route(h, self.router, self.top_k, 1, 1, bias=self.bias, renorm=True)
         return self.ops.moe_experts(h, self.up, self.down, idx, wt, act="swiglu")
+
+
+class CorrectedSigmoidMoE:
+    """Mixture of gated experts behind a sigmoid router with a choice correction: scores s = sigmoid(router . h) (float); experts
+    are CHOSEN by s + correction, inside the `keep` groups (of `groups` equal groups of neighbours) whose two largest corrected
+    scores sum highest; the chosen experts are WEIGHTED by their plain s times `scale` (no division by the chosen scores' sum).  Expert: down .
+    (silu(gate . h) * (up . h)).  An optional shared expert of the same form runs for every token.
+    Returns the list of outputs to be summed ([routed] or [routed, shared]): the caller's residual kernel adds them in one pass."""
+
+    def __init__(self, ops, *, router, correction, gate, up, down, top_k, groups=1, keep=1, scale=1.0, shared=None):
+        """router [E, D], correction [E]; gate / up: lists of E [ff, D]; down: list of E [D, ff]; shared: a GatedFeedForward or None."""
+        self.ops = ops
+        self.router, self.correction = router.contiguous(), correction.float().contiguous()
+        self.up = _interleave(torch.stack(list(gate)), torch.stack(list(up)))          # [E, 2 ff, D]
+        self.down = torch.stack(list(down)).contiguous()
+        E, ff2, D = self.up.shape
+        self.top_k, self.groups, self.keep, self.scale, self.shared = int(top_k), int(groups), int(keep), float(scale), shared
+        if self.router.shape != (E, D) or self.correction.shape != (E,) or self.down.shape != (E, D, ff2 // 2):
+            raise ValueError("mixture of experts: router / expert shapes do not fit each other")
+        if E % self.groups or not 0 < self.keep <= self.groups or not 0 < self.top_k <= self.keep * (E // self.groups):
+            raise ValueError(f"router: {E} experts, {self.groups} groups, keep {self.keep}, top {self.top_k}")
+
+    def __call__(self, h):
+        idx, wt = self.ops.moe_route(h, self.router, self.top_k, self.groups, self.keep, score="sigmoid", correction=self.correction,
+                                     group_top=2, scale=self.scale)
+        y = [self.ops.moe_experts(h, self.up, self.down, idx, wt, act="swiglu")]
+        if self.shared is not None:
+            y.append(self.shared(h))
+        return y

@@ -93,12 +93,16 @@ class HipOps:
 
     attention_split_target = 512        # workgroups a launch of the matrix-core attention should at least have
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0, chunk=None, bias=None):
         """batch: the step's StepBatch (block table, sequence slot and position per token, work tiles).  variant: 0 = the
         matrix-core kernel where it takes the sizes, 1 = always the wave kernel.  key_splits: None = chosen from the number
         of workgroups and the context.  q_first: the caller's promise that every query is zero before that element.
-        pool [rows, R]: one pool for all heads; [G, rows, R]: head h reads pool h // (H / G), all in one launch."""
+        pool [rows, R]: one pool for all heads; [G, rows, R]: head h reads pool h // (H / G), all in one launch.
+        chunk: a query sees only the keys of its own chunk of that many positions.  bias: float [H, n], bias[h, min(i - j, n - 1)]
+        is added to the score of query i and key j."""
         T, H, R = qf.shape
+        assert bias is None or (bias.dtype == torch.float32 and bias.dim() == 2 and bias.size(0) == H and bias.is_contiguous())
+        extra = (int(chunk or 0), 0 if bias is None else bias.data_ptr(), 0 if bias is None else bias.size(1))
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
         self._need(qf, pool, block_table, seq, pos)
@@ -110,6 +114,7 @@ class HipOps:
             # few workgroups and long contexts (decoding): cut the keys over several workgroups, merged by a second launch
             groups = tiles.size(0) * (H // per) * ((per + 31) // 32)
             span = min(batch.max_pos + 1, int(window)) if window else batch.max_pos + 1
+            span = min(span, int(chunk)) if chunk else span
             # (rows wider than 320 elements: one workgroup per CU at a time - a launch of one round of workgroups is the aim)
             target = self.attention_split_target // 2 if R > 320 else self.attention_split_target
             splits = max(1, min(target // max(groups, 1), span // 128, 32)) if key_splits is None else key_splits
@@ -121,11 +126,11 @@ class HipOps:
                                                         block_table.stride(0), pos.data_ptr(), tiles.data_ptr(), tiles.size(0),
                                                         int(window or 0), H, rank, R, page, splits,
                                                         0 if po is None else po.data_ptr(), 0 if pm is None else pm.data_ptr(), T,
-                                                        int(q_first), per, pool_stride, self._s()), "latent_attention_mfma")
+                                                        int(q_first), per, pool_stride, *extra, self._s()), "latent_attention_mfma")
             return out
         self.check(self.L.qsv_latent_attention(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
                                                block_table.stride(0), seq.data_ptr(), pos.data_ptr(), int(window or 0), T, H,
-                                               rank, R, page, per, pool_stride, self.code, variant, self._s()), "latent_attention")
+                                               rank, R, page, per, pool_stride, *extra, self.code, variant, self._s()), "latent_attention")
         return out
 
     def sigmoid_gate(self, o, g):
@@ -194,13 +199,77 @@ class HipOps:
                                             a.size(1), self.code, self._s()), "rms_pair_mean")
         return out
 
-    def glu(self, a):
-        """a [n, 2 ff] with (gate, up) as neighbours -> silu(gate) * up [n, ff]."""
+    GLU_ACTS = {"silu": 0, "gelu_tanh": 1}
+
+    def glu(self, a, act="silu"):
+        """a [n, 2 ff] with (gate, up) as neighbours -> act(gate) * up [n, ff]; act: silu, or gelu_tanh (gelu in its tanh form)."""
         n, ff = a.size(0), a.size(1) // 2
         out = torch.empty((n, ff), dtype=self.dtype, device=a.device)
         self._need(a)
-        self.check(self.L.qsv_glu(out.data_ptr(), a.data_ptr(), n, ff, self.code, self._s()), "glu")
+        self.check(self.L.qsv_glu(out.data_ptr(), a.data_ptr(), n, ff, self.GLU_ACTS[act], self.code, self._s()), "glu")
         return out
+
+    # ---- sinusoidal positions, RMS-normed residual, whole-projection query / key norms ----------------------------------------------
+    def embed_sinusoid(self, tokens, pos, table, freq, scale):
+        """-> float x [T, D] = table[tokens] * scale + the sinusoidal vector of each position (freq float [(D + 1) // 2])."""
+        T, D = tokens.numel(), table.size(1)
+        x = torch.empty((T, D), dtype=torch.float32, device=table.device)
+        self._need(tokens, pos, table, freq)
+        assert freq.dtype == torch.float32 and freq.numel() == (D + 1) // 2
+        self.check(self.L.qsv_embed_sinusoid(x.data_ptr(), table.data_ptr(), tokens.data_ptr(), pos.data_ptr(), freq.data_ptr(),
+                                             float(scale), T, D, self.code, self._s()), "embed_sinusoid")
+        return x
+
+    def add_rms_norm(self, x, ys, w, eps):
+        """x += sum of ys (up to three sublayer outputs, storage type) in place; -> rms_norm(x) * w in the storage type (None if
+        w is None)."""
+        ys = [y for y in ys if y is not None]
+        assert len(ys) <= 3 and all(y.shape == x.shape and y.dtype == self.dtype for y in ys) and x.dtype == torch.float32
+        h = None if w is None else torch.empty(x.shape, dtype=self.dtype, device=x.device)
+        self._need(x, w, *ys)
+        p = [y.data_ptr() for y in ys] + [0] * (3 - len(ys))
+        self.check(self.L.qsv_add_rms_norm(x.data_ptr(), 0 if h is None else h.data_ptr(), *p, 0 if w is None else w.data_ptr(),
+                                           float(eps), x.size(0), x.size(1), self.code, self._s()), "add_rms_norm")
+        return h
+
+    def rms_norm_rows(self, x, rows, w, eps):
+        n = x.size(0) if rows is None else rows.numel()
+        out = torch.empty((n, x.size(1)), dtype=self.dtype, device=x.device)
+        self._need(x, rows, w)
+        self.check(self.L.qsv_rms_norm_rows(out.data_ptr(), x.data_ptr(), 0 if rows is None else rows.data_ptr(), w.data_ptr(),
+                                            float(eps), n, x.size(1), self.code, self._s()), "rms_norm_rows")
+        return out
+
+    def normed_attention_prep(self, proj, q_off, k_off, v_off, heads, kv_heads, dim, vdim, q_w, k_w, eps, scale, v_first, mix, pool,
+                              batch):
+        """-> float queries [T, heads, vdim + dim] = [0 | normed q * scale]; writes the cache rows [v' | normed k] of the step's
+        tokens.  v_first: [T, kv_heads * vdim] (a column slice is fine) or None; mix: the blend's weight on v_first."""
+        T = proj.size(0)
+        qf = torch.empty((T, heads, vdim + dim), dtype=torch.float32, device=proj.device)
+        self._need(proj, q_w, k_w, pool, batch.slot)
+        assert pool.shape[0] == kv_heads and pool.shape[2] == vdim + dim and pool.dtype == self.dtype and proj.dtype == self.dtype
+        assert v_first is None or (v_first.dtype == self.dtype and v_first.stride(1) == 1 and v_first.shape == (T, kv_heads * vdim))
+        self.check(self.L.qsv_normed_attention_prep(qf.data_ptr(), pool.data_ptr(), pool.size(1), proj.data_ptr(), proj.stride(0),
+                                                    q_off, k_off, v_off, heads, kv_heads, dim, vdim, q_w.data_ptr(), k_w.data_ptr(),
+                                                    float(eps), float(scale), 0 if v_first is None else v_first.data_ptr(),
+                                                    0 if v_first is None else v_first.stride(0), float(mix), batch.slot.data_ptr(),
+                                                    T, self.code, self._s()), "normed_attention_prep")
+        return qf
+
+    def max_gates(self, proj, i_off, f_off, bias_i, bias_f, cap, m_state, batch, heads):
+        """Exponential gates with a running maximum from the pre-activations proj[:, i_off : i_off + heads] / [f_off : ...]; m_state
+        float [slots, heads].  -> (decay a, input scale b, maximum m), float [T, heads] each."""
+        T = proj.size(0)
+        a, b, m = (torch.empty((T, heads), dtype=torch.float32, device=proj.device) for _ in range(3))
+        self._need(bias_i, bias_f, m_state)
+        assert proj.stride(1) == 1 and proj.dtype == self.dtype and bias_i.dtype == bias_f.dtype == m_state.dtype == torch.float32
+        assert m_state.shape[1:] == (heads,) and bias_i.numel() == bias_f.numel() == heads
+        runs = batch.runs()
+        el = proj.element_size()
+        self.check(self.L.qsv_max_gates(a.data_ptr(), b.data_ptr(), m.data_ptr(), proj.data_ptr() + i_off * el,
+                                        proj.data_ptr() + f_off * el, proj.stride(0), bias_i.data_ptr(), bias_f.data_ptr(), float(cap),
+                                        m_state.data_ptr(), runs.data_ptr(), runs.size(0), heads, self.code, self._s()), "max_gates")
+        return a, b, m
 
     # ---- attention with rotated keys and values: rotations + cache write ---------------------------------------------------------
     def attention_prep(self, proj, q_off, k_off, v_off, heads, kv_heads, dim, vdim, rot_n, rope_k, rope_v, scale, pool, batch):
@@ -248,41 +317,60 @@ class HipOps:
                                              batch.state_wr.data_ptr(), n_unit, unit_dim, T, self.code, self._s()), "conv_silu_unit")
         return out
 
-    def recurrent_scan(self, q, k, v, decay, beta, state, batch, heads, qk_heads, dim, vdim, q_scale):
+    def recurrent_scan(self, q, k, v, decay, beta, state, batch, heads, qk_heads, dim, vdim, q_scale, kscale=None, v_cols=None):
         """q, k [T, qk_heads * dim], v [T, heads * vdim] (float or storage type, column slices are fine), decay float [T, heads *
-        dim], beta [T, heads] raw (before the sigmoid) or None, state float [slots, heads, dim, vdim] -> o float [T, heads, vdim]."""
+        dim], beta [T, heads] raw (before the sigmoid) or None, state float [slots, heads, dim, vdim] -> o float [T, heads, vdim].
+        decay of shape [T, heads]: one factor per head.  kscale float [T, heads]: multiplies k where it enters the state.
+        v_cols < vdim: v is [T, heads * v_cols] and the state's column v_cols is fed with ones (a normaliser), the rest with zeros."""
         T = q.size(0)
         o = torch.empty((T, heads, vdim), dtype=torch.float32, device=q.device)
-        self._need(decay, state)
+        self._need(decay, state, kscale)
         assert q.dtype == k.dtype == v.dtype and q.stride(1) == k.stride(1) == v.stride(1) == 1
-        assert state.shape[1:] == (heads, dim, vdim) and state.dtype == torch.float32 and decay.shape == (T, heads * dim)
+        head_decay = decay.shape == (T, heads) and dim != 1
+        assert state.shape[1:] == (heads, dim, vdim) and state.dtype == torch.float32 and (head_decay or decay.shape == (T, heads * dim))
+        assert kscale is None or (kscale.dtype == torch.float32 and kscale.shape == (T, heads))
+        assert v.size(1) == heads * (v_cols or vdim)
         runs = batch.runs()
         self.check(self.L.qsv_recurrent_scan(o.data_ptr(), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(),
                                              v.stride(0), dtype_code(q.dtype), decay.data_ptr(),
                                              0 if beta is None else beta.data_ptr(), 0 if beta is None else beta.stride(0),
                                              0 if beta is None else dtype_code(beta.dtype), state.data_ptr(), runs.data_ptr(),
                                              runs.size(0), max(n for _, _, n in batch.items), heads, qk_heads, dim, vdim,
-                                             float(q_scale), self._s()), "recurrent_scan")
+                                             float(q_scale), 0 if kscale is None else kscale.data_ptr(), int(head_decay),
+                                             int(v_cols or 0), self._s()), "recurrent_scan")
         return o
 
-    def head_rms_gate(self, o, w, gate, kind, eps):
-        T, H, dv = o.shape
+    def head_rms_gate(self, o, w, gate, kind, eps, vdim=None, den_m=None):
+        """o float [T, H, n] -> [T, H * vdim] (storage type): per head o[..., :vdim] / its root mean square * w * gate_fn(gate).
+        w [vdim] (shared by the heads) or [H * vdim].  den_m float [T, H] (then n > vdim): the read-out is first divided by
+        max(|o[..., vdim]|, exp(-den_m)) + 1e-6."""
+        T, H, n = o.shape
+        dv = n if vdim is None else vdim
         out = torch.empty((T, H * dv), dtype=self.dtype, device=o.device)
-        self._need(o, w)
+        self._need(o, w, den_m)
         assert gate.stride(1) == 1 and gate.size(1) == H * dv and gate.dtype == self.dtype and w.dtype == self.dtype
+        assert w.numel() in (dv, H * dv) and (den_m is None or (n > dv and den_m.shape == (T, H) and den_m.dtype == torch.float32))
         self.check(self.L.qsv_head_rms_gate(out.data_ptr(), o.data_ptr(), w.data_ptr(), gate.data_ptr(), gate.stride(0),
-                                            {"silu": 0, "sigmoid": 1}[kind], eps, T, H, dv, self.code, self._s()), "head_rms_gate")
+                                            {"silu": 0, "sigmoid": 1}[kind], eps, T, H, dv, n, int(w.numel() != dv),
+                                            0 if den_m is None else den_m.data_ptr(), self.code, self._s()), "head_rms_gate")
         return out
 
-    def moe_route(self, h, router, top_k, groups, keep, bias=None, renorm=False):
+    def moe_route(self, h, router, top_k, groups, keep, bias=None, renorm=False, score="softmax", correction=None, group_top=1,
+                  scale=1.0):
+        """-> (expert indices int32 [T, top_k], weights float [T, top_k]).  score: softmax over all experts, or sigmoid per expert;
+        correction float [E]: added to the scores for the CHOICE only; group_top: a group's score is its largest choice score (1)
+        or the sum of its two largest (2); weights = the chosen experts' scores (renorm: divided by their sum) times scale."""
         T, E = h.size(0), router.size(0)
         idx = torch.empty((T, top_k), dtype=torch.int32, device=h.device)
         wt = torch.empty((T, top_k), dtype=torch.float32, device=h.device)
-        self._need(h, router, bias)
+        self._need(h, router, bias, correction)
         assert bias is None or (bias.dtype == self.dtype and bias.numel() == E)
+        assert correction is None or (correction.dtype == torch.float32 and correction.numel() == E)
         self.check(self.L.qsv_moe_route(idx.data_ptr(), wt.data_ptr(), h.data_ptr(), router.data_ptr(),
                                         0 if bias is None else bias.data_ptr(), int(bool(renorm)), T, h.size(1), E, top_k,
-                                        groups, keep, self.code, self._s()), "moe_route")
+                                        groups, keep, {"softmax": 0, "sigmoid": 1}[score],
+                                        0 if correction is None else correction.data_ptr(), int(group_top), float(scale),
+                                        self.code, self._s()), "moe_route")
         return idx, wt
 
     ACTS = {"none": 0, "relu_sq": 1, "swiglu": 2}
@@ -457,7 +545,7 @@ class TorchOps:
         qr = _rotate(q.view(T, heads, dim + rot_dim)[..., dim:].float(), rope, pos, rot_n)
         return (torch.cat([q_abs.transpose(0, 1).float(), qr], dim=-1) * scale).contiguous()
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0, chunk=None, bias=None):
         T, H, R = qf.shape
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
@@ -467,12 +555,16 @@ class TorchOps:
         for t in range(T):
             p = int(pos[t])
             lo = max(0, p - window + 1) if window else 0
+            if chunk:
+                lo = max(lo, p - p % chunk)
             j = torch.arange(lo, p + 1, device=qf.device)
             at = bt[int(seq[t]), j // page] * page + j % page
             for g, pl in enumerate(pools):
                 rows = pl[at].float()                                                # [n, R]
-                w = torch.softmax(qf[t, g * per:(g + 1) * per] @ rows.t(), dim=-1)   # [per, n]
-                out[t, g * per:(g + 1) * per] = (w @ rows[:, :rank]).to(self.dtype)
+                s = qf[t, g * per:(g + 1) * per] @ rows.t()                          # [per, n]
+                if bias is not None:
+                    s = s + bias[g * per:(g + 1) * per][:, (p - j).clamp(max=bias.size(1) - 1)]
+                out[t, g * per:(g + 1) * per] = (torch.softmax(s, dim=-1) @ rows[:, :rank]).to(self.dtype)
         return out
 
     def sigmoid_gate(self, o, g):
@@ -554,12 +646,19 @@ class TorchOps:
         out[:, :n_unit * unit_dim] = (u / torch.sqrt((u * u).sum(-1, keepdim=True) + 1e-6)).view(-1, n_unit * unit_dim)
         return out
 
-    def recurrent_scan(self, q, k, v, decay, beta, state, batch, heads, qk_heads, dim, vdim, q_scale):
+    def recurrent_scan(self, q, k, v, decay, beta, state, batch, heads, qk_heads, dim, vdim, q_scale, kscale=None, v_cols=None):
         T = q.size(0)
         rep = heads // qk_heads
-        qf = q.float().view(T, qk_heads, dim).repeat_interleave(rep, 1) * q_scale
-        kf = k.float().view(T, qk_heads, dim).repeat_interleave(rep, 1)
-        vf, g = v.float().view(T, heads, vdim), decay.view(T, heads, dim)
+        qf = q.float().reshape(T, qk_heads, dim).repeat_interleave(rep, 1) * q_scale
+        kf = k.float().reshape(T, qk_heads, dim).repeat_interleave(rep, 1)
+        if kscale is not None:
+            kf = kf * kscale[:, :, None]
+        vf = v.float().reshape(T, heads, v_cols or vdim)
+        if v_cols and v_cols < vdim:
+            ones = torch.zeros((T, heads, vdim - v_cols), device=q.device)
+            ones[..., 0] = 1.0
+            vf = torch.cat([vf, ones], dim=-1)
+        g = decay[:, :, None].expand(T, heads, dim) if decay.shape == (T, heads) and dim != 1 else decay.view(T, heads, dim)
         bt = None if beta is None else torch.sigmoid(beta.float())
         o = torch.empty((T, heads, vdim), dtype=torch.float32, device=q.device)
         for slot, first, cnt in batch.items:
@@ -575,35 +674,89 @@ class TorchOps:
             state[slot] = S
         return o
 
-    def head_rms_gate(self, o, w, gate, kind, eps):
-        T, H, dv = o.shape
-        n = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * w.float()
-        g = gate.float().view(T, H, dv)
+    def head_rms_gate(self, o, w, gate, kind, eps, vdim=None, den_m=None):
+        T, H, n_cols = o.shape
+        dv = n_cols if vdim is None else vdim
+        if den_m is not None:
+            o = o[..., :dv] / (torch.maximum(o[..., dv].abs(), torch.exp(-den_m)) + 1e-6)[..., None]
+        o = o[..., :dv]
+        w = w.float().view(H, dv) if w.numel() == H * dv else w.float()
+        n = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * w
+        g = gate.float().reshape(T, H, dv)
         g = g * torch.sigmoid(g) if kind == "silu" else torch.sigmoid(g)
         return (n * g).reshape(T, H * dv).to(self.dtype)
 
     def rms_pair_mean(self, a, wa, b, wb, eps):
         return (0.5 * (self._rms(a, wa, eps) + self._rms(b, wb, eps))).to(self.dtype)
 
-    def glu(self, a):
+    def glu(self, a, act="silu"):
         a = a.float()
         g, u = a[..., 0::2], a[..., 1::2]
-        return (g * torch.sigmoid(g) * u).to(self.dtype)
+        ag = g * torch.sigmoid(g) if act == "silu" else torch.nn.functional.gelu(g, approximate="tanh")
+        return (ag * u).to(self.dtype)
 
-    def moe_route(self, h, router, top_k, groups, keep, bias=None, renorm=False):
+    def moe_route(self, h, router, top_k, groups, keep, bias=None, renorm=False, score="softmax", correction=None, group_top=1,
+                  scale=1.0):
         z = h.float() @ router.float().t()
         if bias is not None:
             z = z + bias.float()
-        if renorm:                                          # weights = softmax over the chosen logits only
+        if renorm and score == "softmax" and correction is None and groups == 1:   # weights = softmax over the chosen logits only
             top = z.topk(top_k, dim=-1)
-            return top.indices.int(), torch.softmax(top.values, dim=-1)
-        s = torch.softmax(z, dim=-1)
+            return top.indices.int(), torch.softmax(top.values, dim=-1) * scale
+        s = torch.softmax(z, dim=-1) if score == "softmax" else torch.sigmoid(z)
+        c = s if correction is None else s + correction.float()
         T, E = s.shape
-        gs = s.view(T, groups, E // groups).amax(-1)
+        per = E // groups
+        gs = c.view(T, groups, per).topk(min(group_top, per), dim=-1).values.sum(-1)
         kept = torch.zeros_like(gs, dtype=torch.bool).scatter_(1, gs.topk(keep, dim=-1).indices, True)
-        ok = kept[:, :, None].expand(T, groups, E // groups).reshape(T, E)
-        idx = s.masked_fill(~ok, -1.0).topk(top_k, dim=-1).indices
-        return idx.int(), s.gather(1, idx)
+        ok = kept[:, :, None].expand(T, groups, per).reshape(T, E)
+        idx = c.masked_fill(~ok, float("-inf")).topk(top_k, dim=-1).indices
+        wt = s.gather(1, idx)
+        if renorm:
+            wt = wt / wt.sum(-1, keepdim=True)
+        return idx.int(), wt * scale
+
+    # ---- sinusoidal positions, RMS-normed residual, whole-projection query / key norms ----------------------------------------------
+    def embed_sinusoid(self, tokens, pos, table, freq, scale):
+        a = pos.float()[:, None] * freq[None, :]                                    # float angles
+        sc = torch.stack([torch.sin(a), torch.cos(a)], dim=-1).reshape(a.size(0), -1)[:, :table.size(1)]
+        return table[tokens.long()].float() * scale + sc
+
+    def add_rms_norm(self, x, ys, w, eps):
+        ys = [y.float() for y in ys if y is not None]
+        if ys:
+            y = ys[0]
+            if len(ys) > 1:
+                y = y + (ys[1] + ys[2] if len(ys) > 2 else ys[1])
+            x += y
+        return None if w is None else self._rms(x, w, eps).to(self.dtype)
+
+    def rms_norm_rows(self, x, rows, w, eps):
+        return self._rms(x if rows is None else x[rows.long()], w, eps).to(self.dtype)
+
+    def normed_attention_prep(self, proj, q_off, k_off, v_off, heads, kv_heads, dim, vdim, q_w, k_w, eps, scale, v_first, mix, pool,
+                              batch):
+        T = proj.size(0)
+        q = self._rms(proj[:, q_off:q_off + heads * dim], q_w, eps).view(T, heads, dim) * scale
+        k = self._rms(proj[:, k_off:k_off + kv_heads * dim], k_w, eps).view(T, kv_heads, dim)
+        v = proj[:, v_off:v_off + kv_heads * vdim].float()
+        if v_first is not None:
+            v = (1.0 - mix) * v + mix * v_first.float()
+        pool[:, batch.slot] = torch.cat([v.view(T, kv_heads, vdim), k], dim=-1).transpose(0, 1).to(self.dtype)
+        return torch.cat([torch.zeros(T, heads, vdim, device=proj.device), q], dim=-1).contiguous()
+
+    def max_gates(self, proj, i_off, f_off, bias_i, bias_f, cap, m_state, batch, heads):
+        li = cap * torch.tanh((proj[:, i_off:i_off + heads].float() + bias_i) / cap)
+        lf = torch.nn.functional.logsigmoid(cap * torch.tanh((proj[:, f_off:f_off + heads].float() + bias_f) / cap))
+        a, b, m = torch.empty_like(li), torch.empty_like(li), torch.empty_like(li)
+        for slot, first, cnt in batch.items:
+            prev = m_state[slot].clone() if int(batch.pos[first]) else torch.zeros_like(m_state[slot])
+            for t in range(first, first + cnt):
+                m[t] = torch.maximum(lf[t] + prev, li[t])
+                a[t], b[t] = torch.exp(lf[t] + prev - m[t]), torch.exp(li[t] - m[t])
+                prev = m[t]
+            m_state[slot] = prev
+        return a, b, m
 
     def moe_experts(self, h, up, down, idx, wt, act="relu_sq"):
         T, D = h.shape

@@ -5,7 +5,11 @@ GatedDeltaRule         S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  
                        g = exp(-exp(A_log) softplus(z + dt_bias)) per head and key channel, beta = sigmoid(.) per head,
                        q, k, v through a short causal convolution + silu, q and k made unit vectors per head
 
-Both read every projection of the layer input from ONE product; the low-rank second stages (decay, gate) are products of
+MatrixLSTM             S <- a S + b k v^T, n <- a n + b k;  o = S^T q / (max(|n . q|, exp(-m)) + 1e-6)
+                       a = exp(f + m' - m), b = exp(i - m) per head from a log input gate i and a log forget gate f, both soft-
+                       capped, and the running maximum m = max(f + m', i) that keeps the exponentials in range (m' = 0 at the start)
+
+All read every projection of the layer input from ONE product; the low-rank second stages (decay, gate) are products of
 their own.  State per sequence: the matrices (one copy: a run of tokens is read, advanced and written back by the workgroups
 that own its columns) and, for the convolution, the last taps - 1 inputs (two copies, swapped per step).
 """
@@ -93,3 +97,33 @@ class ParallelMixer:
         a = self.left(h, batch, pools[:self._np], states[:self._ns])
         b = self.right(h, batch, pools[self._np:], states[self._ns:])
         return self.ops.rms_pair_mean(a, self.w_left, b, self.w_right, self.eps)
+
+
+class MatrixLSTM:
+    """Matrix memory with exponential gates (mLSTM).  The normaliser n rides along as one more column of the state: the values
+    are extended by a column of ones, so S' = [S | n] [dim, vdim + pad] obeys the same recurrence and q reads S^T q and n . q
+    in one go.  State per sequence: S' and the running maximum m per head."""
+
+    def __init__(self, ops, *, heads, dim, vdim, gate_cap, eps, weights):
+        """weights: q, k [H dim, D], v, g [H vdim, D], o [D, H vdim], norm [H vdim], i, f [H, D], i_b, f_b [H]."""
+        self.ops, self.H, self.dim, self.vdim, self.cap, self.eps = ops, heads, dim, vdim, float(gate_cap), float(eps)
+        w = weights
+        D = w["q"].size(1)
+        _check(w, {"q": (heads * dim, D), "k": (heads * dim, D), "v": (heads * vdim, D), "g": (heads * vdim, D), "o": (D, heads * vdim),
+                   "norm": (heads * vdim,), "i": (heads, D), "f": (heads, D), "i_b": (heads,), "f_b": (heads,)}, "matrix LSTM")
+        if self.cap <= 0.0:
+            raise ValueError(f"matrix LSTM: gate cap {gate_cap}")
+        self.w_in = torch.cat([w["q"], w["k"], w["v"], w["g"], w["i"], w["f"]], dim=0).contiguous()
+        self.b_i, self.b_f = w["i_b"].float().contiguous(), w["f_b"].float().contiguous()
+        self.norm, self.w_o = w["norm"].contiguous(), w["o"].contiguous()
+        self.cols = vdim + (4 if vdim % 4 == 0 else 1)             # (a multiple of four keeps the kernels' 16-byte accesses)
+        self.cache_rows, self.state_specs = [], [StateSpec((heads, dim, self.cols)), StateSpec((heads,))]
+
+    def __call__(self, h, batch, pools, states, carry=None):
+        ops, H, d, dv = self.ops, self.H, self.dim, self.vdim
+        proj = linear(h, self.w_in)
+        o_k, o_v, o_g, o_i = H * d, 2 * H * d, 2 * H * d + H * dv, 2 * H * d + 2 * H * dv
+        a, b, m = ops.max_gates(proj, o_i, o_i + H, self.b_i, self.b_f, self.cap, states[1], batch, H)
+        o = ops.recurrent_scan(proj[:, :o_k], proj[:, o_k:o_v], proj[:, o_v:o_g], a, None, states[0], batch, H, H, d, self.cols,
+                               d ** -0.5, kscale=b, v_cols=dv)
+        return linear(ops.head_rms_gate(o, self.norm, proj[:, o_g:o_i], "sigmoid", self.eps, vdim=dv, den_m=m), self.w_o)

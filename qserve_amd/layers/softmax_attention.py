@@ -8,7 +8,13 @@ dimensions of every q and k head turn with the position (halves layout, table `r
 Cache: per key / value head one pool of rows [v (vdim) | k (dim)].  The attention itself is the paged row-attention kernel of
 the latent layers (qserve_amd.layers.latent_attention): a query [0 (vdim) | q * scale] against such rows scores q . k, and
 the softmax-weighted sum of the rows' first vdim elements is the output; one launch serves all key / value heads.
+
+`NormedChunkAttention` is the position-free sibling on the same cache rows and kernel: queries and keys are RMS-normed over the
+whole projection, positions enter through a learned bias per (distance bucket, head) and through chunks that bound what a query
+sees, and the values may be blended with those an earlier layer computed for the same token.
 """
+import math
+
 import torch
 
 from .ops import linear
@@ -38,4 +44,78 @@ class RotatedValueAttention:
                                 self.rope_k.reserve(n), self.rope_v.reserve(n), self.scale, pool, batch)
         o = ops.latent_attention(qf, pool, batch, None, self.vdim, self.page, q_first=self.vdim)      # head h reads pool h // (H / G)
         ops.rotate_heads(o, self.rope_v.table, batch.pos, -1.0)
+        return linear(o.view(T, H * self.vdim), self.w_o)
+
+
+def distance_bucket(n, rows, far):
+    """Row of a bias table with `rows` rows for the distance n >= 0: distances below rows / 2 have a row each; from there the rows
+    are spaced evenly in log(distance) up to `far`, bucket = rows / 2 + floor(log(n / half) / log(far / half) * (rows - half)), capped
+    at the last row.  With integer `far` the floor is taken exactly (integer powers), not through floating-point logarithms."""
+    half = rows // 2
+    if n < half:
+        return n
+    m = rows - half
+    if far <= half:
+        raise ValueError(f"a bias table of {rows} rows needs its far distance above {half}, not {far}")
+    if float(far).is_integer():
+        far, k = int(far), 0
+        while k < m and far ** (k + 1) * half ** (m - k - 1) <= n ** m:     # (far / half)^((k + 1) / m) <= n / half
+            k += 1
+    else:
+        k = int(math.floor(math.log(n / half) / math.log(far / half) * m))
+    return min(rows - 1, half + k)
+
+
+def distance_bias_table(rel, far, length):
+    """rel [rows, H] -> float [H, length]: entry [h, n] = rel[distance_bucket(n), h]; the kernels clamp larger distances to the
+    last entry, so `length` = far + 1 covers every distance (beyond `far` the bucket is the last row)."""
+    rows = rel.size(0)
+    idx = torch.tensor([distance_bucket(n, rows, far) for n in range(length)], dtype=torch.long, device=rel.device)
+    return rel.float()[idx].t().contiguous()
+
+
+class NormedChunkAttention:
+    def __init__(self, ops, *, heads, kv_heads, dim, vdim, scale, eps, weights, chunk=None, bias_far=None, mix=None, publish=False,
+                 page=64):
+        """weights: q [H dim, D], k [G dim, D], v [G vdim, D], q_norm [H dim], k_norm [G dim], o [D, H vdim], rel [rows, H] or None.
+        chunk: position i sees j <= i with floor(j / chunk) == floor(i / chunk) (None: all j <= i).  bias_far: the distance at
+        which the bias table's logarithmic rows end.  publish: this layer's own values go into the step's carry as "v_first";
+        mix (a number): the cached values are (1 - mix) v + mix carry["v_first"]."""
+        if heads % kv_heads:
+            raise ValueError(f"attention: {heads} heads over {kv_heads}")
+        self.ops, self.H, self.G, self.dim, self.vdim, self.page = ops, heads, kv_heads, dim, vdim, page
+        self.scale, self.eps, self.chunk, self.mix, self.publish = float(scale), float(eps), int(chunk) if chunk else None, mix, publish
+        w = weights
+        D = w["q"].size(1)
+        for k, shp in {"q": (heads * dim, D), "k": (kv_heads * dim, D), "v": (kv_heads * vdim, D), "q_norm": (heads * dim,),
+                       "k_norm": (kv_heads * dim,), "o": (D, heads * vdim)}.items():
+            if tuple(w[k].shape) != shp:
+                raise ValueError(f"attention weight {k}: shape {tuple(w[k].shape)}, expected {shp}")
+        self.w_in, self.w_o = torch.cat([w["q"], w["k"], w["v"]], dim=0).contiguous(), w["o"].contiguous()
+        self.q_norm, self.k_norm = w["q_norm"].contiguous(), w["k_norm"].contiguous()
+        self.bias = None
+        if w.get("rel") is not None:
+            if w["rel"].dim() != 2 or w["rel"].size(1) != heads or bias_far is None:
+                raise ValueError(f"attention bias table {tuple(w['rel'].shape)} for {heads} heads, far distance {bias_far}")
+            far = int(bias_far) if float(bias_far).is_integer() else float(bias_far)
+            length = int(math.ceil(far)) + 1
+            self.bias = distance_bias_table(w["rel"], far, min(length, self.chunk) if self.chunk else length)
+        self.cache_rows, self.state_specs = [(kv_heads, vdim + dim)], []
+
+    def __call__(self, h, batch, pools, states, carry=None):
+        ops, T, H, G = self.ops, h.size(0), self.H, self.G
+        pool = pools[0]                                                    # [G, rows, vdim + dim]
+        proj = linear(h, self.w_in)
+        o_k, o_v = H * self.dim, (H + G) * self.dim
+        own = proj[:, o_v:o_v + G * self.vdim]
+        v_first = None
+        if self.mix is not None:
+            v_first = carry["v_first"]
+            if v_first.shape != own.shape:
+                raise ValueError("blended values: the layers' value sizes differ")
+        if self.publish:
+            carry["v_first"] = own
+        qf = ops.normed_attention_prep(proj, 0, o_k, o_v, H, G, self.dim, self.vdim, self.q_norm, self.k_norm, self.eps, self.scale,
+                                       v_first, self.mix or 0.0, pool, batch)
+        o = ops.latent_attention(qf, pool, batch, None, self.vdim, self.page, q_first=self.vdim, chunk=self.chunk, bias=self.bias)
         return linear(o.view(T, H * self.vdim), self.w_o)
