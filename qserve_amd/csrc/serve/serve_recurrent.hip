@@ -438,7 +438,7 @@ __global__ __launch_bounds__(64) void max_gates_kernel(float* __restrict__ a_out
         float prev = __shfl_up(m, 1, 64);
         if (lane == 0) prev = carry;
         if (ok) {
-            a_out[t * H + h] = expf(lf + prev - m);
+            a_out[t * H + h] = expf(lf + (prev - m));            // (prev - m is exact; lf + prev would round lf away)
             b_out[t * H + h] = expf(li - m);
             m_out[t * H + h] = m;
         }

@@ -753,7 +753,7 @@ class TorchOps:
             prev = m_state[slot].clone() if int(batch.pos[first]) else torch.zeros_like(m_state[slot])
             for t in range(first, first + cnt):
                 m[t] = torch.maximum(lf[t] + prev, li[t])
-                a[t], b[t] = torch.exp(lf[t] + prev - m[t]), torch.exp(li[t] - m[t])
+                a[t], b[t] = torch.exp(lf[t] + (prev - m[t])), torch.exp(li[t] - m[t])
                 prev = m[t]
             m_state[slot] = prev
         return a, b, m
