@@ -134,6 +134,14 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
         __syncthreads();
         if (k0 + Z * BN <= p_last) issue(k0 + Z * BN);
         if (!active || (ti % S) != sp || k0 > wp_last || k0 + BN - 1 < wlo) continue;   // (wave-uniform)
+        // the bias of this lane's eight (query, key) pairs: requested before the score product, added after it
+        float bv[2][4];
+        if (brow) {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) bv[mt][r] = brow[min(max(p_row - (k0 + 16 * mt + 4 * g4 + r), 0), bias_len - 1)];
+        }
         // ---- S^T = K Q^T: two blocks of 16 keys; this lane gets keys 16 mt + 4 g4 + r of its own query row ----
         v4f sacc[2] = {v4f{0.f, 0.f, 0.f, 0.f}, v4f{0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
@@ -154,7 +162,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
             for (int r = 0; r < 4; ++r) {
                 const int key = k0 + 16 * mt + 4 * g4 + r;
                 const bool vis = key <= p_row && key >= lo_row;
-                if (brow && vis) sacc[mt][r] += brow[min(p_row - key, bias_len - 1)];
+                if (brow) sacc[mt][r] += bv[mt][r];
                 sacc[mt][r] = vis ? sacc[mt][r] : -INFINITY;
                 tmax = fmaxf(tmax, sacc[mt][r]);
             }

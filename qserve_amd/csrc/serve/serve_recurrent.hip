@@ -105,8 +105,9 @@ __device__ __forceinline__ float4 ld4(const bf16_t* p, size_t i) {
 
 // VEC: dim, vdim, the row strides and the operands' addresses are multiples of four elements - staged four at a time.
 // R rows and NC columns of the state per lane (with NC > 1 the token's k, q and decay rows are read from LDS once for NC columns).
-template <typename TQ, typename TB, bool DELTA, bool VEC, int R, int NC>
-__global__ __launch_bounds__(256) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
+// OCC: waves per SIMD the register allocation must leave room for (1: no demand - the compiler takes about 230 registers, two waves).
+template <typename TQ, typename TB, bool DELTA, bool VEC, int R, int NC, int OCC>
+__global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restrict__ o, const TQ* __restrict__ q, int64_t q_stride,
                                                              const TQ* __restrict__ k, int64_t k_stride, const TQ* __restrict__ v,
                                                              int64_t v_stride, const float* __restrict__ decay,
                                                              const TB* __restrict__ beta, int64_t beta_stride,
@@ -565,6 +566,12 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     while (lpc8 * 8 < dim) lpc8 <<= 1;
     const int64_t waves8 = (int64_t)n_runs * heads * (((int64_t)vdim * lpc8 + 63) / 64);
     const int R = dim <= 64 * 8 && waves8 <= 2560 ? 8 : 16, NC = 1;
+    // The 8-row form takes about 230 registers: two four-wave workgroups per CU, and a launch of more than 2 x 256 of them runs in
+    // rounds, each as long as a full one (132 columns instead of 128 at 8 x 16 (run, head) pairs: 0.94 ms instead of 0.49).  Where a
+    // third workgroup per CU saves a round, the variant compiled for three waves per SIMD is used.
+    const int cols8 = 64 / lpc8, wpb8 = (vdim + cols8 - 1) / cols8 >= 4 ? 4 : (vdim + cols8 - 1) / cols8 > 1 ? 2 : 1;
+    const int64_t groups8 = (int64_t)n_runs * heads * ((vdim + wpb8 * cols8 - 1) / (wpb8 * cols8)) * wpb8 / 4;
+    const bool three = R == 8 && !beta && (groups8 + 767) / 768 < (groups8 + 511) / 512;
     QSV_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dim > 0 && dim <= 64 * 16 && vdim > 0 && n_runs >= 0 &&
                     heads <= 65535,
                 "qsv_recurrent_scan: bad sizes (%d heads over %d, state %d x %d)", heads, qk_heads, dim, vdim);
@@ -592,16 +599,17 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     const bool vec = dim % 4 == 0 && vdim % 4 == 0 && v_cols % 4 == 0 && VB % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 &&
                      (uintptr_t)q % (4 * el) == 0 && (uintptr_t)k % (4 * el) == 0 && (uintptr_t)v % (4 * el) == 0 &&
                      (uintptr_t)decay % 16 == 0;
-#define QSV_SCAN_V(TQ, TB, DELTA, VEC, RR, CC)                                                                               \
-    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, VEC, RR, CC>), grid, block, lds, (hipStream_t)stream, o,            \
+#define QSV_SCAN_V(TQ, TB, DELTA, VEC, RR, CC, OC)                                                                              \
+    hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, VEC, RR, CC, OC>), grid, block, lds, (hipStream_t)stream, o,        \
                        (const TQ*)q, q_stride, (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta,         \
                        beta_stride, state, runs, heads, qk_heads, dim, vdim, lpc_log, CT, q_scale, kscale, head_decay, v_cols)
 #define QSV_SCAN(TQ, TB, DELTA)                                \
     do {                                                       \
-        if (vec && R == 8) QSV_SCAN_V(TQ, TB, DELTA, true, 8, 1);   \
-        else if (R == 8) QSV_SCAN_V(TQ, TB, DELTA, false, 8, 1);    \
-        else if (vec) QSV_SCAN_V(TQ, TB, DELTA, true, 16, 1);       \
-        else QSV_SCAN_V(TQ, TB, DELTA, false, 16, 1);               \
+        if (vec && R == 8 && three && !DELTA) QSV_SCAN_V(TQ, TB, false, true, 8, 1, 3);   \
+        else if (vec && R == 8) QSV_SCAN_V(TQ, TB, DELTA, true, 8, 1, 1);   \
+        else if (R == 8) QSV_SCAN_V(TQ, TB, DELTA, false, 8, 1, 1);    \
+        else if (vec) QSV_SCAN_V(TQ, TB, DELTA, true, 16, 1, 1);       \
+        else QSV_SCAN_V(TQ, TB, DELTA, false, 16, 1, 1);               \
     } while (0)
     if (beta) {
         if (qkv_dtype == QSV_F32 && beta_dtype == QSV_F32) QSV_SCAN(float, float, true);

@@ -264,10 +264,77 @@ __global__ __launch_bounds__(NT) void add_rms_norm_kernel(float* __restrict__ x,
     const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
     for (int i = threadIdx.x; i < D; i += NT) st(h, t * D + i, x[t * D + i] * inv * ld(w, i));   // (this thread's own writes)
 }
+// The same for widths that are multiples of four, up to 4 * NT * VPT: 16-byte accesses of the stream (8-byte of bfloat16 rows), the
+// row stays in registers between the sum of squares and the scaling.
+__device__ __forceinline__ float4 ld4v(const float* p, size_t i) { return *(const float4*)(p + i); }
+__device__ __forceinline__ float4 ld4v(const bf16_t* p, size_t i) {
+    const uint2 u = *(const uint2*)(p + i);
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u), __uint_as_float(u.y << 16),
+                       __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void st4v(float* p, size_t i, float4 v) { *(float4*)(p + i) = v; }
+__device__ __forceinline__ void st4v(bf16_t* p, size_t i, float4 v) {
+    uint2 u;
+    u.x = (uint32_t)f2bf(v.x) | ((uint32_t)f2bf(v.y) << 16);
+    u.y = (uint32_t)f2bf(v.z) | ((uint32_t)f2bf(v.w) << 16);
+    *(uint2*)(p + i) = u;
+}
+template <typename T, int VPT>
+__global__ __launch_bounds__(NT) void add_rms_norm_vec_kernel(float* __restrict__ x, T* __restrict__ h, const T* __restrict__ a,
+                                                              const T* __restrict__ b, const T* __restrict__ c,
+                                                              const T* __restrict__ w, float eps, int D) {
+    __shared__ float red[NT / 64 + 1];
+    const size_t t = blockIdx.x;
+    float4 v[VPT];
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int i = (threadIdx.x + k * NT) * 4;
+        if (i >= D) continue;
+        v[k] = ld4v(x, t * D + i);
+        if (a || b || c) {
+            float4 y = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (b) y = ld4v(b, t * D + i);
+            if (c) {
+                const float4 z = ld4v(c, t * D + i);
+                y.x += z.x; y.y += z.y; y.z += z.z; y.w += z.w;
+            }
+            if (a) {
+                const float4 z = ld4v(a, t * D + i);
+                y.x = z.x + y.x; y.y = z.y + y.y; y.z = z.z + y.z; y.w = z.w + y.w;
+            }
+            v[k].x += y.x; v[k].y += y.y; v[k].z += y.z; v[k].w += y.w;
+            st4v(x, t * D + i, v[k]);
+        }
+        s += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+    }
+    if (!h) return;
+    const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int i = (threadIdx.x + k * NT) * 4;
+        if (i >= D) continue;
+        const float4 g = ld4v(w, i);
+        st4v(h, t * D + i, make_float4(v[k].x * inv * g.x, v[k].y * inv * g.y, v[k].z * inv * g.z, v[k].w * inv * g.w));
+    }
+}
 extern "C" int qsv_add_rms_norm(float* x, void* h, const void* a, const void* b, const void* c, const void* w, float eps, int n,
                                 int D, int dtype, void* stream) {
     QSV_REQUIRE(x && n >= 0 && D > 0 && (!h || w), "qsv_add_rms_norm: bad arguments");
     if (n == 0) return QSV_OK;
+    const int vecs = (D / 4 + NT - 1) / NT;
+    if (D % 4 == 0 && vecs <= 8) {
+#define QSV_ARN(V)                                                                                                                 \
+    QSV_DISPATCH(dtype, "qsv_add_rms_norm",                                                                                        \
+                 hipLaunchKernelGGL((add_rms_norm_vec_kernel<T, V>), dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (T*)h, (const T*)a, \
+                                    (const T*)b, (const T*)c, (const T*)w, eps, D))
+        if (vecs <= 1) QSV_ARN(1);
+        else if (vecs <= 2) QSV_ARN(2);
+        else if (vecs <= 4) QSV_ARN(4);
+        else QSV_ARN(8);
+#undef QSV_ARN
+        return qsv_launch_status("qsv_add_rms_norm");
+    }
     QSV_DISPATCH(dtype, "qsv_add_rms_norm",
                  hipLaunchKernelGGL(add_rms_norm_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (T*)h, (const T*)a, (const T*)b,
                                     (const T*)c, (const T*)w, eps, D));

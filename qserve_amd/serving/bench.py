@@ -2,6 +2,7 @@
 
     python bench.py --design vekalorn [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside the W4A8KV4 Llama engine
     python bench.py --design mumelix  [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside Vekalorn
+    python bench.py --design vepolix  [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside Mumelix
 
 Per size (random weights, 4 layers, vocabulary 32000): prompt phase = 8 prompts x 1024 tokens in one step through
 Engine.execute; decoding = 64 sequences at context 1024, one token each per step.  Beside them the Llama-style W4A8KV4
@@ -75,7 +76,8 @@ class OpTimer:
     """HIP events around every call of the ops object's methods and of the vendor products (one step at a time)."""
     NAMES = ("embed", "add_layer_norm", "layer_norm_rows", "latent_prep", "latent_query", "latent_attention", "sigmoid_gate",
              "moe_route", "moe_experts", "embed_streams", "hc_read", "hc_write", "dyt_sum_rows", "rms_pair_mean", "glu",
-             "attention_prep", "rotate_heads", "decay", "conv_silu_unit", "recurrent_scan", "head_rms_gate")
+             "attention_prep", "rotate_heads", "decay", "conv_silu_unit", "recurrent_scan", "head_rms_gate", "embed_sinusoid",
+             "add_rms_norm", "rms_norm_rows", "normed_attention_prep", "max_gates")
 
     def __init__(self, ops):
         self.ops, self.events, self.calls, self.on = ops, [], [], False
@@ -90,7 +92,7 @@ class OpTimer:
         import importlib
         return [importlib.import_module("qserve_amd." + m) for m in
                 ("layers.latent_attention", "layers.moe", "layers.recurrent", "layers.softmax_attention", "models.vekalorn",
-                 "models.mumelix")]
+                 "models.mumelix", "models.vepolix")]
 
     def _wrap(self, name, fn):
         def timed(*a, **k):
@@ -402,6 +404,135 @@ def bench_mumelix(name, s, dev, steps, warmup):
     return out
 
 
+# ---- Vepolix ----------------------------------------------------------------------------------------------------------------
+def vepolix_config(s, m):
+    """Mumelix's sizes in Vepolix's layers: attention with the same heads and cache rows (chunks longer than the workload's
+    contexts, so both attend over the same keys), a matrix memory of the gated-linear-attention state's size, the same experts
+    (plus a shared one) on the recurrent layers and a dense unit of the active expert width on the attention layers."""
+    a = {"type": "attention", "mlp": {"kind": "dense", "ff": s["top"] * s["ff"]},
+         "mixer": {"heads": m["a_heads"], "kv_heads": m["a_kv"], "dim": m["a_dim"], "vdim": m["a_vdim"], "mask": {"size": 2048},
+                   "bias_max": 1024, "scale": 1.0 / math.sqrt(m["a_dim"]), "v_mix": True}}
+    r = {"type": "mlstm", "mixer": {"heads": m["g_heads"], "dim": m["g_dim"], "vdim": m["g_vdim"], "gate_cap": 20.0},
+         "mlp": {"kind": "moe", "expert": {"ff": s["ff"]}, "shared": {"ff": s["ff"]},
+                 "router": {"experts": s["experts"], "top": s["top"], "scale": 2.0, "groups": {"count": s["groups"], "keep": s["keep"]}}}}
+    return {"architecture": "Vepolix", "width": s["width"], "vocab": VOCAB, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+            "layers": [a, r, a, r][:LAYERS]}
+
+
+def vepolix_weights(cfg, dev, seed=0, bias_rows=32):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    D, V = cfg["width"], cfg["vocab"]
+
+    def mat(o, i, s=1.0):
+        return (torch.randn((o, i), device=dev, generator=g) * (s / math.sqrt(i))).bfloat16()
+
+    def vec(n, mean=1.0, s=0.1):
+        return (mean + s * torch.randn((n,), device=dev, generator=g)).bfloat16()
+
+    def unit(p, ff):
+        W[p + "gate"], W[p + "up"], W[p + "down"] = mat(ff, D), mat(ff, D), mat(D, ff)
+
+    W = {"embed": torch.randn((V, D), device=dev, generator=g).bfloat16(), "head": mat(V, D), "final.norm": vec(D)}
+    for i, L in enumerate(cfg["layers"]):
+        p, x = f"l{i}.", L["mixer"]
+        W[p + "norm1"] = vec(D)
+        q = p + "mix."
+        if L["type"] == "attention":
+            H, G, d, dv = x["heads"], x["kv_heads"], x["dim"], x["vdim"]
+            W.update({q + "q": mat(H * d, D), q + "k": mat(G * d, D), q + "v": mat(G * dv, D), q + "o": mat(D, H * dv), q + "q.norm": vec(H * d),
+                      q + "k.norm": vec(G * d), q + "rel": vec(bias_rows * H, 0.0, 1.0).view(bias_rows, H), q + "vmix": torch.tensor(0.3).bfloat16()})
+        else:
+            H, d, dv = x["heads"], x["dim"], x["vdim"]
+            W.update({q + "q": mat(H * d, D), q + "k": mat(H * d, D), q + "v": mat(H * dv, D), q + "g": mat(H * dv, D), q + "o": mat(D, H * dv),
+                      q + "norm": vec(H * dv), q + "i": mat(H, D), q + "i.b": vec(H, 0.0, 1.0), q + "f": mat(H, D), q + "f.b": vec(H, 3.0, 1.0)})
+        mlp, q = L["mlp"], p + "mlp."
+        if mlp["kind"] == "dense":
+            unit(q, mlp["ff"])
+        else:
+            for e in range(mlp["router"]["experts"]):
+                unit(f"{q}e{e}.", mlp["expert"]["ff"])
+            unit(q + "shared.", mlp["shared"]["ff"])
+            W[q + "router"], W[q + "correction"] = mat(mlp["router"]["experts"], D, 3.0), vec(mlp["router"]["experts"], 0.0, 0.1)
+    return W
+
+
+def bench_vepolix(name, s, dev, steps, warmup):
+    from ..models.vepolix import Vepolix
+    from .engine import Engine
+    m = MUMELIX[name]
+    cfg = vepolix_config(s, m)
+    NB, L, BP = 64, 1024, 8
+    eng = Engine(Vepolix, cfg, vepolix_weights(cfg, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 384), max_seqs=NB)
+    timer = OpTimer(eng.ops)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, VOCAB, (L,), generator=g).tolist() for _ in range(NB)]
+    slots = [eng.open_sequence() for _ in range(NB)]
+    small = ("latent_attention", "add_rms_norm", "normed_attention_prep", "max_gates", "head_rms_gate", "recurrent_scan")
+    pre_ms, ops_pre, rep_pre = [], None, {}
+    for i in range(0, NB, BP):
+        items = [(slots[j], prompts[j]) for j in range(i, i + BP)]
+        want = [k * L + L - 1 for k in range(BP)]
+        if i == BP:                                          # one step with events around every launch
+            ops_pre, _ = timer.step(lambda: eng.execute(items, want))
+            rep_pre = {k: timer.replay(k, 3) for k in small if k != "recurrent_scan" and k != "max_gates"}   # (these two advance state)
+            continue
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.execute(items, want)
+        torch.cuda.synchronize()
+        if i > 0:
+            pre_ms.append((time.perf_counter() - t0) * 1e3)
+    pre = sorted(pre_ms)[len(pre_ms) // 2]
+    nxt = [[int(torch.randint(0, VOCAB, (1,), generator=g))] for _ in range(NB)]
+    want = list(range(NB))
+
+    def decode():
+        eng.execute([(slots[j], nxt[j]) for j in range(NB)], want)
+
+    dec_eager = timed(decode, steps, warmup)
+    ops_dec, dec_events_ms = timer.step(decode)
+    rep_dec = {k: timer.replay(k, 20) for k in ("latent_attention", "moe_experts", "add_rms_norm", "normed_attention_prep", "head_rms_gate")}
+    eng.decode_graphs = True
+    dec = timed(decode, steps, warmup)
+    graph_ok = any(v is not False for v in eng._graphs.values()) and bool(eng._graphs)
+    ctx = eng.cache.length[slots[0]]
+    T, D = BP * L, s["width"]
+    n_att = sum(1 for x in cfg["layers"] if x["type"] == "attention")
+    n_rec = LAYERS - n_att
+    R = m["a_dim"] + m["a_vdim"]
+    att_flops = n_att * BP * sum(p + 1 for p in range(L)) * m["a_heads"] * (m["a_dim"] + m["a_vdim"]) * 2.0
+    att_pre = att_flops / (rep_pre["latent_attention"] * 1e-3) / 1e12
+    att_bytes = n_att * NB * ctx * m["a_kv"] * R * 2.0
+    att_dec = att_bytes / (rep_dec["latent_attention"] * 1e-3) / 1e9
+    # recurrence: 5 float operations per state element and token (decay, k v, add; q S, add); decoding moves the state twice
+    el = n_rec * m["g_heads"] * m["g_dim"] * m["g_vdim"]
+    scan_pre = T * 5.0 * el / (ops_pre["recurrent_scan"] * 1e-3) / 1e12
+    scan_dec = NB * el * 4.0 * 2 / (ops_dec["recurrent_scan"] * 1e-3) / 1e9
+    moe_flops = n_rec * T * s["top"] * 3 * 2.0 * s["ff"] * D
+    moe_pre = moe_flops / (ops_pre["moe_experts"] * 1e-3) / 1e12
+    moe_bytes = n_rec * min(s["experts"], NB * s["top"]) * 3 * s["ff"] * D * 2.0
+    moe_dec = moe_bytes / (rep_dec["moe_experts"] * 1e-3) / 1e9
+    # residual kernel: reads and writes the float stream, reads the sublayers' outputs (2 on attention layers, 3 on the others),
+    # writes the next input; the first call only norms, the last only adds
+    res_bytes = T * (LAYERS * (8.0 * D + 2.0 * D) + (2 * n_att + 3 * n_rec) * 2.0 * D)
+    res_pre = res_bytes / (rep_pre["add_rms_norm"] * 1e-3) / 1e9
+    out = dict(model=f"Vepolix-{name}", sizes=m, prefill_tokens_per_s=T / pre * 1e3, prefill_ms=pre, decode_tokens_per_s=NB / dec * 1e3,
+               decode_ms=dec, decode_from_hipgraph=graph_ok, decode_ms_eager=dec_eager, decode_ms_gpu_events=dec_events_ms, context=ctx,
+               prefill_ops_ms=ops_pre, decode_ops_ms=ops_dec, prefill_kernels_ms=rep_pre, decode_kernels_ms=rep_dec,
+               roofline=dict(prefill_attention_tflops=att_pre, prefill_attention_frac_bf16_peak=att_pre / BF16_PEAK_TFLOPS,
+                             decode_attention_gbs=att_dec, decode_attention_frac_hbm=att_dec / HBM_PEAK_GBS,
+                             prefill_experts_tflops=moe_pre, prefill_experts_frac_bf16_peak=moe_pre / BF16_PEAK_TFLOPS,
+                             decode_experts_gbs=moe_dec, decode_experts_frac_hbm=moe_dec / HBM_PEAK_GBS,
+                             prefill_recurrence_tflops=scan_pre, prefill_recurrence_frac_fp32_valu_peak=scan_pre / FP32_VALU_PEAK_TFLOPS,
+                             decode_recurrence_gbs=scan_dec, decode_recurrence_frac_hbm=scan_dec / HBM_PEAK_GBS,
+                             prefill_residual_kernel_gbs=res_pre, prefill_residual_kernel_frac_hbm=res_pre / HBM_PEAK_GBS))
+    for sl in slots:
+        eng.close_sequence(sl)
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
 def main(args, helpers):
     dev = "cuda:0"
     torch.cuda.set_device(0)
@@ -411,12 +542,15 @@ def main(args, helpers):
         build.build(verbose=False)
     steps, warmup = min(args.steps, 32), min(args.warmup, 8)
     for name in args.design_sizes.split(","):
-        if args.design == "mumelix" and name not in MUMELIX:      # (sizes that differ in a Vekalorn-only constant)
+        if args.design in ("mumelix", "vepolix") and name not in MUMELIX:      # (sizes that differ in a Vekalorn-only constant)
             continue
         s = SIZES[name]
         line = {"design": args.design, "size": name, "sizes": s, "layers": LAYERS, "vocab": VOCAB, "dtype": "bf16",
                 "data": "synthetic", "workload": "prefill 8 x 1024 tokens in one step; decode 64 sequences at context 1024"}
-        if args.design == "mumelix":
+        if args.design == "vepolix":
+            line["vepolix"] = bench_vepolix(name, s, dev, steps, warmup)
+            line["mumelix"] = bench_mumelix(name, s, dev, steps, warmup)
+        elif args.design == "mumelix":
             line["mumelix"] = bench_mumelix(name, s, dev, steps, warmup)
             line["vekalorn"] = bench_vekalorn(name, s, dev, steps, warmup)
         else:
