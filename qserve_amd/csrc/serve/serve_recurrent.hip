@@ -115,6 +115,8 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
                                                              int QH, int dim, int vdim, int lpc_log, int CT, float q_scale,
                                                              const float* __restrict__ kscale, int head_decay, int v_cols) {
     static_assert(R == 4 || R == 8 || R == 16, "rows per lane");
+    // (the three-wave variant stages half as many tokens per chunk: fewer prefetch registers and deferred read-outs, no spills)
+    constexpr int MAX_CT = OCC >= 3 ? SCAN_CT / 2 : SCAN_CT, PFK = OCC >= 3 ? SCAN_PFK / 2 : SCAN_PFK, PFV = OCC >= 3 ? SCAN_PFV / 2 : SCAN_PFV;
     extern __shared__ __attribute__((aligned(16))) float sm[];
     const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wave = tid >> 6, nw = nthr >> 6;
     const int lpc = 1 << lpc_log, cols = 64 >> lpc_log;                           // cols: column groups (of NC) per wave
@@ -134,13 +136,13 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
 #pragma unroll
         for (int i = 0; i < R; ++i) S[c][i] = (!fresh && j + c < vdim && r0 + i < dim) ? Sg[(size_t)(r0 + i) * vdim + j + c] : 0.f;
 
-    float pk[SCAN_PFK], pv[SCAN_PFV], pb = 0.f;
+    float pk[PFK], pv[PFV], pb = 0.f;
     // requests the operands of tokens [c0, c0 + ct) of the run into registers
     auto fetch = [&](int c0, int ct) {
         const int nk = ct * 3 * DIMP, nv = ct * VB;
         if (VEC) {
 #pragma unroll
-            for (int i = 0; i < SCAN_PFK / 4; ++i) {
+            for (int i = 0; i < PFK / 4; ++i) {
                 const int idx = (tid + i * nthr) * 4;
                 float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (idx < nk) {
@@ -164,7 +166,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
                 pk[4 * i] = val.x; pk[4 * i + 1] = val.y; pk[4 * i + 2] = val.z; pk[4 * i + 3] = val.w;
             }
 #pragma unroll
-            for (int i = 0; i < SCAN_PFV / 4; ++i) {
+            for (int i = 0; i < PFV / 4; ++i) {
                 const int idx = (tid + i * nthr) * 4;
                 float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
                 if (idx < nv) {
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < SCAN_PFK; ++i) {
+            for (int i = 0; i < PFK; ++i) {
                 const int idx = tid + i * nthr;
                 float val = 0.f;
                 if (idx < nk) {
@@ -190,7 +192,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
                 pk[i] = val;
             }
 #pragma unroll
-            for (int i = 0; i < SCAN_PFV; ++i) {
+            for (int i = 0; i < PFV; ++i) {
                 const int idx = tid + i * nthr;
                 float val = 0.f;
                 if (idx < nv) {
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
         const int nk = ct * 3 * DIMP, nv = ct * VB;
         if (VEC) {
 #pragma unroll
-            for (int i = 0; i < SCAN_PFK / 4; ++i) {
+            for (int i = 0; i < PFK / 4; ++i) {
                 const int idx = (tid + i * nthr) * 4;
                 if (idx < nk) {
                     const int tt = (idx >> dimp_log) / 3;
@@ -215,7 +217,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
                 }
             }
 #pragma unroll
-            for (int i = 0; i < SCAN_PFV / 4; ++i) {
+            for (int i = 0; i < PFV / 4; ++i) {
                 const int idx = (tid + i * nthr) * 4;
                 if (idx < nv) {
                     const int tt = idx >> vb_log;
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < SCAN_PFK; ++i) {
+            for (int i = 0; i < PFK; ++i) {
                 const int idx = tid + i * nthr;
                 if (idx < nk) {
                     const int tt = (idx >> dimp_log) / 3;
@@ -232,7 +234,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
                 }
             }
 #pragma unroll
-            for (int i = 0; i < SCAN_PFV; ++i) {
+            for (int i = 0; i < PFV; ++i) {
                 const int idx = tid + i * nthr;
                 if (idx < nv) {
                     const int tt = idx >> vb_log;
@@ -250,9 +252,9 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
         stage(ct);
         __syncthreads();
         if (c0 + CT < n) fetch(c0 + CT, min(CT, n - c0 - CT));   // in flight while this chunk is computed
-        float oacc[SCAN_CT][NC];
+        float oacc[MAX_CT][NC];
 #pragma unroll
-        for (int tt = 0; tt < SCAN_CT; ++tt) {
+        for (int tt = 0; tt < MAX_CT; ++tt) {
 #pragma unroll
             for (int c = 0; c < NC; ++c) oacc[tt][c] = 0.f;
             if (tt >= ct) continue;                              // (uniform)
@@ -305,7 +307,7 @@ __global__ __launch_bounds__(256, OCC) void recurrent_scan_kernel(float* __restr
             }
         }
 #pragma unroll
-        for (int tt = 0; tt < SCAN_CT; ++tt)
+        for (int tt = 0; tt < MAX_CT; ++tt)
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 const float sum = column_sum(oacc[tt][c], lpc);
@@ -565,13 +567,30 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     int lpc8 = 1;
     while (lpc8 * 8 < dim) lpc8 <<= 1;
     const int64_t waves8 = (int64_t)n_runs * heads * (((int64_t)vdim * lpc8 + 63) / 64);
-    const int R = dim <= 64 * 8 && waves8 <= 2560 ? 8 : 16, NC = 1;
-    // The 8-row form takes about 230 registers: two four-wave workgroups per CU, and a launch of more than 2 x 256 of them runs in
-    // rounds, each as long as a full one (132 columns instead of 128 at 8 x 16 (run, head) pairs: 0.94 ms instead of 0.49).  Where a
-    // third workgroup per CU saves a round, the variant compiled for three waves per SIMD is used.
-    const int cols8 = 64 / lpc8, wpb8 = (vdim + cols8 - 1) / cols8 >= 4 ? 4 : (vdim + cols8 - 1) / cols8 > 1 ? 2 : 1;
-    const int64_t groups8 = (int64_t)n_runs * heads * ((vdim + wpb8 * cols8 - 1) / (wpb8 * cols8)) * wpb8 / 4;
-    const bool three = R == 8 && !beta && (groups8 + 767) / 768 < (groups8 + 511) / 512;
+    int R = dim <= 64 * 8 && waves8 <= 2560 ? 8 : 16;
+    const int NC = 1;
+    // Both forms take about 230 registers: two four-wave workgroups of the 8-row form (one of the 16-row form) per CU, and a launch
+    // of more workgroups than that runs in rounds, each as long as a full one (132 columns instead of 128 at 8 x 16 (run, head)
+    // pairs: 0.94 ms instead of 0.49).  A third form - 8 rows, compiled for three waves per SIMD, half the staging - holds three
+    // workgroups per CU at 1.23 times the round's length; it is taken where that saves rounds (costs in rounds of the 8-row form).
+    bool three = false;
+    if (!beta && dim <= 64 * 8) {
+        const int cols8 = 64 / lpc8, wpb8 = (vdim + cols8 - 1) / cols8 >= 4 ? 4 : (vdim + cols8 - 1) / cols8 > 1 ? 2 : 1;
+        const int64_t pairs = (int64_t)n_runs * heads;
+        const int64_t groups8 = pairs * ((vdim + wpb8 * cols8 - 1) / (wpb8 * cols8)) * wpb8 / 4;
+        const int cols16 = cols8 * 2 > 64 ? 64 : cols8 * 2;
+        const int64_t groups16 = pairs * ((vdim + 4 * cols16 - 1) / (4 * cols16));
+        const double legacy = R == 8 ? (double)((groups8 + 511) / 512) : 1.12 * (double)((groups16 + 255) / 256);
+        const double lean = 1.23 * (double)((groups8 + 767) / 768);
+        const size_t el8 = qkv_dtype == QSV_F32 ? 4 : 2;         // (the third form has 16-byte staging only)
+        const bool vec8 = dim % 4 == 0 && vdim % 4 == 0 && v_cols % 4 == 0 && (wpb8 * cols8) % 4 == 0 && q_stride % 4 == 0 &&
+                          k_stride % 4 == 0 && v_stride % 4 == 0 && (uintptr_t)q % (4 * el8) == 0 && (uintptr_t)k % (4 * el8) == 0 &&
+                          (uintptr_t)v % (4 * el8) == 0 && (uintptr_t)decay % 16 == 0;
+        if (vec8 && lean < legacy) {
+            three = true;
+            R = 8;
+        }
+    }
     QSV_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dim > 0 && dim <= 64 * 16 && vdim > 0 && n_runs >= 0 &&
                     heads <= 65535,
                 "qsv_recurrent_scan: bad sizes (%d heads over %d, state %d x %d)", heads, qk_heads, dim, vdim);
@@ -586,26 +605,28 @@ extern "C" int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, con
     int nw = 1;
     while (nw < 4 && nw < waves_needed) nw <<= 1;
     const int VB = nw * cols * NC, nthr = nw * 64;
-    int CT = SCAN_CT;                                            // tokens per staged chunk: what the prefetch registers and 48 KiB hold
-    while (CT > 1 && ((CT * 3 * DIMP + nthr - 1) / nthr > SCAN_PFK || (CT * VB + nthr - 1) / nthr > SCAN_PFV ||
-                      (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4 > 48 * 1024))
-        CT >>= 1;
-    QSV_REQUIRE((CT * 3 * DIMP + nthr - 1) / nthr <= SCAN_PFK && (CT * VB + nthr - 1) / nthr <= SCAN_PFV,
-                "qsv_recurrent_scan: a state of %d rows does not fit the staging registers", dim);
-    const size_t lds = (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4;
-    const dim3 grid(n_runs, heads, (vdim + VB - 1) / VB), block(nthr);
-    QSV_REQUIRE(grid.z <= 65535, "qsv_recurrent_scan: too many column blocks");
     const size_t el = qkv_dtype == QSV_F32 ? 4 : 2;
     const bool vec = dim % 4 == 0 && vdim % 4 == 0 && v_cols % 4 == 0 && VB % 4 == 0 && q_stride % 4 == 0 && k_stride % 4 == 0 && v_stride % 4 == 0 &&
                      (uintptr_t)q % (4 * el) == 0 && (uintptr_t)k % (4 * el) == 0 && (uintptr_t)v % (4 * el) == 0 &&
                      (uintptr_t)decay % 16 == 0;
+    const bool lean = three && vec;                              // (the variant for three waves per SIMD: half the staging)
+    const int max_ct = lean ? SCAN_CT / 2 : SCAN_CT, pfk = lean ? SCAN_PFK / 2 : SCAN_PFK, pfv = lean ? SCAN_PFV / 2 : SCAN_PFV;
+    int CT = max_ct;                                             // tokens per staged chunk: what the prefetch registers and 48 KiB hold
+    while (CT > 1 && ((CT * 3 * DIMP + nthr - 1) / nthr > pfk || (CT * VB + nthr - 1) / nthr > pfv ||
+                      (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4 > 48 * 1024))
+        CT >>= 1;
+    QSV_REQUIRE((CT * 3 * DIMP + nthr - 1) / nthr <= pfk && (CT * VB + nthr - 1) / nthr <= pfv,
+                "qsv_recurrent_scan: a state of %d rows does not fit the staging registers", dim);
+    const size_t lds = (size_t)CT * (3 * DIMP + ((VB + 4) & ~3)) * 4;
+    const dim3 grid(n_runs, heads, (vdim + VB - 1) / VB), block(nthr);
+    QSV_REQUIRE(grid.z <= 65535, "qsv_recurrent_scan: too many column blocks");
 #define QSV_SCAN_V(TQ, TB, DELTA, VEC, RR, CC, OC)                                                                              \
     hipLaunchKernelGGL((recurrent_scan_kernel<TQ, TB, DELTA, VEC, RR, CC, OC>), grid, block, lds, (hipStream_t)stream, o,        \
                        (const TQ*)q, q_stride, (const TQ*)k, k_stride, (const TQ*)v, v_stride, decay, (const TB*)beta,         \
                        beta_stride, state, runs, heads, qk_heads, dim, vdim, lpc_log, CT, q_scale, kscale, head_decay, v_cols)
 #define QSV_SCAN(TQ, TB, DELTA)                                \
     do {                                                       \
-        if (vec && R == 8 && three && !DELTA) QSV_SCAN_V(TQ, TB, false, true, 8, 1, 3);   \
+        if (lean && !DELTA) QSV_SCAN_V(TQ, TB, false, true, 8, 1, 3);   \
         else if (vec && R == 8) QSV_SCAN_V(TQ, TB, DELTA, true, 8, 1, 1);   \
         else if (R == 8) QSV_SCAN_V(TQ, TB, DELTA, false, 8, 1, 1);    \
         else if (vec) QSV_SCAN_V(TQ, TB, DELTA, true, 16, 1, 1);       \

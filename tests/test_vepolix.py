@@ -741,3 +741,41 @@ def test_decode_steps_from_a_graph_match_eager_steps(dtype, std):
         assert_close(got[1][k], got[0][k], tol, f"graph against eager, sequence {k}")
         if dtype == "float32":
             assert_close(got[1][k], ref[k][:got[0][k].shape[0]], F32_TOL, f"graph against the oracle, sequence {k}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("runs,heads,dim,vdim,cols", [(32, 4, 64, 128, 132), (8, 16, 64, 128, 132), (8, 32, 64, 128, 132), (3, 2, 64, 128, 132),
+                                                      (32, 4, 32, 64, 68), (20, 8, 64, 128, 128)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["float32", "bfloat16"])
+def test_scan_forms_at_launch_sizes_that_fill_the_chip(runs, heads, dim, vdim, cols, dtype):
+    """The scan kernel picks its form (rows per lane, waves per SIMD, staging depth) from the number of workgroups a launch has;
+    small models never reach the forms for full chips.  Runs of unequal lengths, some continuing a sequence, with one decay per
+    head, a key scale and the column of ones, against the unfused statement of the same recurrence."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    dev = "cuda:0"
+    g = torch.Generator().manual_seed(runs * 100 + heads)
+    lens = [int(n) for n in torch.randint(1, 41, (runs,), generator=g)]
+    lens[0], lens[-1] = 40, 17
+    T = sum(lens)
+    items, pos, at = [], [], 0
+    for s, n in enumerate(lens):
+        items.append((s, at, n))
+        first = 0 if s % 3 else 5                                            # every third run continues a sequence
+        pos += range(first, first + n)
+        at += n
+    pos = torch.tensor(pos, dtype=torch.int32, device=dev)
+    batch = StepBatch(tokens=None, seq=None, pos=pos, slot=None, block_table=None, max_pos=int(pos.max()), n_tokens=T, items=items)
+    proj = (torch.randn(T, 2 * heads * dim + heads * vdim, generator=g) * 0.5).to(dtype).to(dev)
+    q, k, v = proj[:, :heads * dim], proj[:, heads * dim:2 * heads * dim], proj[:, 2 * heads * dim:]
+    decay = (torch.rand(T, heads, generator=g) * 0.3 + 0.7).to(dev)
+    ks = torch.rand(T, heads, generator=g).to(dev)
+    state = torch.randn(runs, heads, dim, cols, generator=g).to(dev)
+    kw = dict(kscale=ks, v_cols=vdim) if cols > vdim else {}
+    outs = []
+    for name in ("hip", "unfused"):
+        st = state.clone()
+        o = make_ops(name, dtype, dev).recurrent_scan(q, k, v, decay, None, st, batch, heads, heads, dim, cols, dim ** -0.5, **kw)
+        outs.append((o.double().cpu(), st.double().cpu()))
+    assert_close(outs[0][0], outs[1][0], 2e-5, "read-outs")
+    assert_close(outs[0][1], outs[1][1], 2e-5, "states")
