@@ -61,7 +61,7 @@ class Vepolix:
                 wm["rel"] = w(p + "rel") if (p + "rel") in weights else None
                 blend = bool(m.get("v_mix"))
                 mixer = NormedChunkAttention(
-                    ops, heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                    ops, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m["vdim"]),
                     scale=float(m["scale"]), eps=eps, weights=wm, chunk=int(m["mask"]["size"]) if m.get("mask") else None,
                     bias_far=m.get("bias_max"), publish=blend and not published,
                     mix=float(weights[p + "vmix"].float()) if blend and published else None, page=page)
