@@ -97,3 +97,41 @@ class CorrectedSigmoidMoE:
         if self.shared is not None:
             y.append(self.shared(h))
         return y
+
+
+class ReluSquaredFeedForward:
+    """Dense feed-forward without a gate: down . relu(up . h)^2, no biases."""
+
+    def __init__(self, ops, *, up, down):
+        if down.shape != (up.size(1), up.size(0)):
+            raise ValueError("feed-forward: up / down shapes do not fit each other")
+        self.ops, self.w_up, self.w_down = ops, up.contiguous(), down.contiguous()
+
+    def __call__(self, h):
+        from .ops import linear
+        return linear(self.ops.relu_sq(linear(h, self.w_up)), self.w_down)
+
+
+class IdentityExpertMoE:
+    """Mixture of clamped gated experts and identity experts behind a softmax router with a choice correction.  Scores s =
+    softmax(router . h) over ALL router outputs (float); the `top_k` outputs with the largest s + correction are chosen and
+    weighted by their plain s (no renormalisation).  The last `identity` router outputs have no tensors: their expert returns its
+    input.  The others: g = min(gate . h, limit), u = clamp(up . h, -limit, limit), down . (g sigmoid(1.702 g) (u + 1))."""
+
+    def __init__(self, ops, *, router, correction, gate, up, down, top_k, identity=0, limit):
+        """router [E + identity, D], correction [E + identity]; gate / up: lists of E [ff, D]; down: list of E [D, ff]."""
+        self.ops = ops
+        self.router, self.correction = router.contiguous(), correction.float().contiguous()
+        self.up = _interleave(torch.stack(list(gate)), torch.stack(list(up)))          # [E, 2 ff, D]
+        self.down = torch.stack(list(down)).contiguous()
+        E, ff2, D = self.up.shape
+        self.top_k, self.identity, self.limit = int(top_k), int(identity), float(limit)
+        n = E + self.identity
+        if self.router.shape != (n, D) or self.correction.shape != (n,) or self.down.shape != (E, D, ff2 // 2) or self.identity < 0:
+            raise ValueError("mixture of experts: router / expert shapes do not fit each other")
+        if not 0 < self.top_k <= n:
+            raise ValueError(f"router: {n} outputs, top {self.top_k}")
+
+    def __call__(self, h):
+        idx, wt = self.ops.moe_route(h, self.router, self.top_k, 1, 1, correction=self.correction)
+        return self.ops.moe_experts(h, self.up, self.down, idx, wt, act="clamped_glu", limit=self.limit)

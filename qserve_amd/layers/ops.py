@@ -93,19 +93,31 @@ class HipOps:
 
     attention_split_target = 512        # workgroups a launch of the matrix-core attention should at least have
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0, chunk=None, bias=None):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0, chunk=None, bias=None,
+                         keep_first=0, sink=None, pooled=None, pool_block=0):
         """batch: the step's StepBatch (block table, sequence slot and position per token, work tiles).  variant: 0 = the
         matrix-core kernel where it takes the sizes, 1 = always the wave kernel.  key_splits: None = chosen from the number
         of workgroups and the context.  q_first: the caller's promise that every query is zero before that element.
         pool [rows, R]: one pool for all heads; [G, rows, R]: head h reads pool h // (H / G), all in one launch.
         chunk: a query sees only the keys of its own chunk of that many positions.  bias: float [H, n], bias[h, min(i - j, n - 1)]
-        is added to the score of query i and key j."""
+        is added to the score of query i and key j.  keep_first: the first that many positions of the sequence stay visible
+        behind the window.  sink float [H]: exp(sink[h]) joins the softmax's denominator (no key, no value).  pooled (shaped like
+        pool, ceil(page / pool_block) rows per page, written by `pool_blocks`): one more key / value row per block of pool_block
+        positions that lies wholly before the window."""
         T, H, R = qf.shape
+        assert sink is None or (sink.dtype == torch.float32 and sink.numel() == H and sink.is_contiguous())
+        assert pooled is None or (window and pool_block > 0 and bias is None and not chunk and not keep_first and pooled.dim() == pool.dim()
+                                  and pooled.dtype == pool.dtype and pooled.size(-1) == R)
+        assert not keep_first or (window and not chunk)
+        per_page = (page + pool_block - 1) // pool_block if pooled is not None else 0
+        assert pooled is None or pooled.size(-2) == pool.size(-2) // page * per_page
+        more = (int(keep_first or 0), 0 if sink is None else sink.data_ptr(), 0 if pooled is None else pooled.data_ptr(),
+                0 if pooled is None or pooled.dim() == 2 else pooled.stride(0), int(pool_block) if pooled is not None else 0, per_page)
         assert bias is None or (bias.dtype == torch.float32 and bias.dim() == 2 and bias.size(0) == H and bias.is_contiguous())
         extra = (int(chunk or 0), 0 if bias is None else bias.data_ptr(), 0 if bias is None else bias.size(1))
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
-        self._need(qf, pool, block_table, seq, pos)
+        self._need(qf, pool, block_table, seq, pos, pooled)
         assert pool.size(-1) == R and block_table.dtype == torch.int32 and seq.dtype == torch.int32
         per, pool_stride = (H, 0) if pool.dim() == 2 else (H // pool.size(0), pool.stride(0))
         assert pool.dim() == 2 or H % pool.size(0) == 0
@@ -115,6 +127,7 @@ class HipOps:
             groups = tiles.size(0) * (H // per) * ((per + 31) // 32)
             span = min(batch.max_pos + 1, int(window)) if window else batch.max_pos + 1
             span = min(span, int(chunk)) if chunk else span
+            span += int(keep_first or 0) + (batch.max_pos // pool_block if pooled is not None else 0)
             # (rows wider than 320 elements: one workgroup per CU at a time - a launch of one round of workgroups is the aim)
             target = self.attention_split_target // 2 if R > 320 else self.attention_split_target
             splits = max(1, min(target // max(groups, 1), span // 128, 32)) if key_splits is None else key_splits
@@ -126,11 +139,12 @@ class HipOps:
                                                         block_table.stride(0), pos.data_ptr(), tiles.data_ptr(), tiles.size(0),
                                                         int(window or 0), H, rank, R, page, splits,
                                                         0 if po is None else po.data_ptr(), 0 if pm is None else pm.data_ptr(), T,
-                                                        int(q_first), per, pool_stride, *extra, self._s()), "latent_attention_mfma")
+                                                        int(q_first), per, pool_stride, *extra, *more, self._s()), "latent_attention_mfma")
             return out
         self.check(self.L.qsv_latent_attention(out.data_ptr(), qf.data_ptr(), pool.data_ptr(), block_table.data_ptr(),
                                                block_table.stride(0), seq.data_ptr(), pos.data_ptr(), int(window or 0), T, H,
-                                               rank, R, page, per, pool_stride, *extra, self.code, variant, self._s()), "latent_attention")
+                                               rank, R, page, per, pool_stride, *extra, *more, self.code, variant, self._s()),
+                   "latent_attention")
         return out
 
     def sigmoid_gate(self, o, g):
@@ -199,14 +213,15 @@ class HipOps:
                                             a.size(1), self.code, self._s()), "rms_pair_mean")
         return out
 
-    GLU_ACTS = {"silu": 0, "gelu_tanh": 1}
+    GLU_ACTS = {"silu": 0, "gelu_tanh": 1, "clamped": 2}
 
-    def glu(self, a, act="silu"):
-        """a [n, 2 ff] with (gate, up) as neighbours -> act(gate) * up [n, ff]; act: silu, or gelu_tanh (gelu in its tanh form)."""
+    def glu(self, a, act="silu", limit=0.0):
+        """a [n, 2 ff] with (gate, up) as neighbours -> act(gate) * up [n, ff]; act: silu, gelu_tanh (gelu in its tanh form), or
+        clamped: g = min(gate, limit), u = clamp(up, -limit, limit) -> g sigmoid(1.702 g) (u + 1)."""
         n, ff = a.size(0), a.size(1) // 2
         out = torch.empty((n, ff), dtype=self.dtype, device=a.device)
         self._need(a)
-        self.check(self.L.qsv_glu(out.data_ptr(), a.data_ptr(), n, ff, self.GLU_ACTS[act], self.code, self._s()), "glu")
+        self.check(self.L.qsv_glu(out.data_ptr(), a.data_ptr(), n, ff, self.GLU_ACTS[act], float(limit), self.code, self._s()), "glu")
         return out
 
     # ---- sinusoidal positions, RMS-normed residual, whole-projection query / key norms ----------------------------------------------
@@ -292,6 +307,81 @@ class HipOps:
                    "rotate_heads")
         return o
 
+
+    # ---- sandwich norms, sink / kept-first / pooled-block attention, element-wise gated recurrence -----------------------------------
+    def add_normed_rms_norm(self, x, y, w_post, w_next, eps):
+        """x += rms_norm(y) * w_post in place (y None: nothing is added); -> rms_norm(x) * w_next in the storage type (None if
+        w_next is None).  The weights hold one number (a gain for all coordinates) or one per coordinate."""
+        T, D = x.shape
+        h = None if w_next is None else torch.empty((T, D), dtype=self.dtype, device=x.device)
+        self._need(x, y, w_post, w_next)
+        assert x.dtype == torch.float32 and (y is None or (y.shape == x.shape and y.dtype == self.dtype and w_post is not None))
+        for w in (w_post, w_next):
+            assert w is None or (w.dtype == self.dtype and w.numel() in (1, D))
+        self.check(self.L.qsv_add_normed_rms_norm(x.data_ptr(), 0 if h is None else h.data_ptr(), 0 if y is None else y.data_ptr(),
+                                                  0 if y is None else w_post.data_ptr(), int(y is not None and w_post.numel() != 1),
+                                                  0 if w_next is None else w_next.data_ptr(),
+                                                  int(w_next is not None and w_next.numel() != 1), float(eps), T, D, self.code,
+                                                  self._s()), "add_normed_rms_norm")
+        return h
+
+    def relu_sq(self, a):
+        """a <- relu(a)^2 in place."""
+        self._need(a)
+        self.check(self.L.qsv_relu_sq(a.data_ptr(), a.numel(), self.code, self._s()), "relu_sq")
+        return a
+
+    def qk_norm_rope_prep(self, q, k, v, heads, kv_heads, dim, vdim, q_w, k_w, per_head, eps, rope, rot_n, scale, pool, batch):
+        """q [T, heads * dim], k [T, kv_heads * dim], v [T, kv_heads * vdim] (float or storage type, column slices are fine; k and v
+        None: the layer caches nothing).  Queries and keys are RMS-normed per head (weight [dim], shared by the heads) or over the
+        whole projection (weight as wide as it), then the first rot_n dimensions of every head turn with the position (pairs of
+        neighbours; rope float [positions, 2, rot_n / 2] or None).  -> float queries [T, heads, vdim + dim] = [0 | q * scale];
+        writes the cache rows [v | k] of the step's tokens into pool [kv_heads, rows, vdim + dim]."""
+        T = q.size(0)
+        qf = torch.empty((T, heads, vdim + dim), dtype=torch.float32, device=q.device)
+        self._need(q_w, k_w, rope, pool, batch.slot, batch.pos)
+        assert q.stride(1) == 1 and q.size(1) == heads * dim and q_w.dtype == self.dtype and q_w.numel() == (dim if per_head else heads * dim)
+        assert rope is None or (rope.dtype == torch.float32 and rope.size(-1) * 2 == rot_n and rot_n <= dim and rope.size(0) > batch.max_pos)
+        kp = [0, 0, 0, 0, 0, 0, 0]
+        if k is not None:
+            assert k.dtype == v.dtype == q.dtype and k.stride(1) == v.stride(1) == 1 and k.size(1) == kv_heads * dim
+            assert v.size(1) == kv_heads * vdim and k_w.dtype == self.dtype and k_w.numel() == (dim if per_head else kv_heads * dim)
+            assert pool.shape[0] == kv_heads and pool.shape[2] == vdim + dim and pool.dtype == self.dtype
+            kp = [k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), k_w.data_ptr(), pool.data_ptr(), pool.size(1)]
+        self.check(self.L.qsv_qk_norm_rope_prep(qf.data_ptr(), q.data_ptr(), q.stride(0), *kp[:4], dtype_code(q.dtype), heads, kv_heads,
+                                                dim, vdim, q_w.data_ptr(), kp[4], int(bool(per_head)), float(eps),
+                                                0 if rope is None else rope.data_ptr(), int(rot_n if rope is not None else 0),
+                                                float(scale), kp[5], kp[6], batch.slot.data_ptr(), batch.pos.data_ptr(), T, self.code,
+                                                self._s()), "qk_norm_rope_prep")
+        return qf
+
+    def pool_blocks(self, pool, pooled, batch, block, page):
+        """For every token of the step that completes a block of `block` positions: the mean of the block's cache rows (as the pool
+        holds them) goes into `pooled` [kv_heads, pages * ceil(page / block), row]: the block that starts in page p at offset o
+        has row p * ceil(page / block) + o // block."""
+        per_page = (page + block - 1) // block
+        self._need(pool, pooled, batch.block_table, batch.seq, batch.pos)
+        assert pool.dim() == 3 and pooled.dim() == 3 and pooled.size(0) == pool.size(0) and pooled.size(2) == pool.size(2)
+        assert pooled.size(1) == pool.size(1) // page * per_page and pooled.dtype == pool.dtype == self.dtype
+        self.check(self.L.qsv_pool_blocks(pooled.data_ptr(), pooled.size(1), pool.data_ptr(), pool.size(1), batch.block_table.data_ptr(),
+                                          batch.block_table.stride(0), batch.seq.data_ptr(), batch.pos.data_ptr(), batch.n_tokens,
+                                          pool.size(0), pool.size(2), int(block), int(page), per_page, self.code, self._s()),
+                   "pool_blocks")
+
+    def min_gru_scan(self, proj, z_off, x_off, g_off, b_z, b_x, state, batch, width):
+        """Element-wise gated recurrence S <- (1 - z) S + z c with z = sigmoid(proj[:, z_off ..] + b_z), c = u + 1/2 (u >= 0) or
+        sigmoid(u) (u < 0), u = proj[:, x_off ..] + b_x; state float [slots, width].  -> S * silu(proj[:, g_off ..]) [T, width]."""
+        T = proj.size(0)
+        out = torch.empty((T, width), dtype=self.dtype, device=proj.device)
+        self._need(b_z, b_x, state)
+        assert proj.stride(1) == 1 and proj.dtype == self.dtype and b_z.dtype == b_x.dtype == self.dtype and state.dtype == torch.float32
+        assert state.shape[1:] == (width,) and b_z.numel() == b_x.numel() == width and max(z_off, x_off, g_off) + width <= proj.size(1)
+        runs = batch.runs()
+        self.check(self.L.qsv_min_gru_scan(out.data_ptr(), proj.data_ptr(), proj.stride(0), z_off, x_off, g_off, b_z.data_ptr(),
+                                           b_x.data_ptr(), state.data_ptr(), runs.data_ptr(), runs.size(0), width, self.code,
+                                           self._s()), "min_gru_scan")
+        return out
+
     # ---- recurrences ----------------------------------------------------------------------------------------------------------
     def decay(self, z, bias, a_log, tau, heads, dim):
         """z [T, heads * dim] (storage type; a column slice is fine) -> float decays: a_log given: exp(-exp(a_log[h]) softplus(z +
@@ -305,7 +395,10 @@ class HipOps:
                                     float(tau), T, heads, dim, self.code, self._s()), "decay")
         return out
 
-    def conv_silu_unit(self, proj, off, conv_w, hist, batch, n_unit, unit_dim):
+    def conv_silu_unit(self, proj, off, conv_w, hist, batch, n_unit, unit_dim, act="silu"):
+        """Causal convolution over time of the columns [off, off + C) of proj with per-channel taps conv_w [C, taps], then silu
+        (act "none": nothing), then the first n_unit groups of unit_dim channels made unit vectors.  hist: two-copy state, the last
+        taps - 1 inputs of every sequence.  -> float [T, C]."""
         T = proj.size(0)
         C, taps = conv_w.shape
         out = torch.empty((T, C), dtype=torch.float32, device=proj.device)
@@ -314,7 +407,8 @@ class HipOps:
         assert hist.size(1) == max(taps - 1, 1)
         self.check(self.L.qsv_conv_silu_unit(out.data_ptr(), proj.data_ptr(), proj.stride(0), off, C, taps, conv_w.data_ptr(),
                                              hist.data_ptr(), batch.run_off.data_ptr(), batch.state_rd.data_ptr(),
-                                             batch.state_wr.data_ptr(), n_unit, unit_dim, T, self.code, self._s()), "conv_silu_unit")
+                                             batch.state_wr.data_ptr(), n_unit, unit_dim, {"none": 0, "silu": 1}[act], T, self.code, self._s()),
+                   "conv_silu_unit")
         return out
 
     def recurrent_scan(self, q, k, v, decay, beta, state, batch, heads, qk_heads, dim, vdim, q_scale, kscale=None, v_cols=None):
@@ -373,30 +467,31 @@ class HipOps:
                                         self.code, self._s()), "moe_route")
         return idx, wt
 
-    ACTS = {"none": 0, "relu_sq": 1, "swiglu": 2}
+    ACTS = {"none": 0, "relu_sq": 1, "swiglu": 2, "clamped_glu": 3}
 
-    def moe_experts(self, h, up, down, idx, wt, act="relu_sq"):
+    def moe_experts(self, h, up, down, idx, wt, act="relu_sq", limit=0.0):
         """up [E, rows, D], down [E, D, ff]; y[t] = sum_k wt[t, k] * down[idx[t, k]] a(up[idx[t, k]] h[t]).  act "relu_sq":
-        a = relu(.)^2, rows = ff; "swiglu": up's rows come in pairs (2f = gate, 2f + 1 = up), a_f = silu(gate_f) up_f, rows = 2 ff."""
+        a = relu(.)^2, rows = ff; "swiglu": up's rows come in pairs (2f = gate, 2f + 1 = up), a_f = silu(gate_f) up_f, rows = 2 ff;
+        "clamped_glu": the same pairs with g = min(gate_f, limit), u = clamp(up_f, -limit, limit), a_f = g sigmoid(1.702 g) (u + 1).
+        Indices at or above E (up.size(0)) name identity experts: their output is h[t] itself."""
         T, D = h.shape
         top_k, rows = idx.size(1), up.size(1)
         a = self.ACTS[act]
-        ff = rows // 2 if a == 2 else rows
+        ff = rows // 2 if a >= 2 else rows
         if (self.code == BF16 and self.moe_token_slots < T * top_k <= self.moe_expert_major_slots and D % 8 == 0 and ff % 8 == 0
                 and D <= 4096 and ff <= 4096):
-            return self._moe_experts_expert_major(h, up, down, idx, wt, a)
+            return self._moe_experts_expert_major(h, up, down, idx, wt, a, limit)
         if T * top_k > self.moe_sorted_above:
-            return self._moe_experts_sorted(h, up, down, idx, wt, a)
+            return self._moe_experts_sorted(h, up, down, idx, wt, a, limit)
         act = torch.empty((T, top_k, ff), dtype=self.dtype, device=h.device)
         y = torch.empty((T, D), dtype=self.dtype, device=h.device)
         self._need(h, up, down, idx, wt)
         assert up.shape[2] == D and down.shape == (up.size(0), D, ff)
-        self.check(self.L.qsv_moe_up(act.data_ptr(), h.data_ptr(), up.data_ptr(), idx.data_ptr(), T, top_k, D, rows, a, self.code,
-                                     self._s()), "moe_up")
+        self.check(self.L.qsv_moe_up(act.data_ptr(), h.data_ptr(), up.data_ptr(), idx.data_ptr(), T, top_k, D, rows, a, float(limit),
+                                     up.size(0), self.code, self._s()), "moe_up")
         self.check(self.L.qsv_moe_down(y.data_ptr(), act.data_ptr(), down.data_ptr(), idx.data_ptr(), wt.data_ptr(), T, top_k, D,
-                                       ff, self.code, self._s()), "moe_down")
+                                       ff, h.data_ptr(), up.size(0), self.code, self._s()), "moe_down")
         return y
-
 
     # More (token, expert) slots than this: sort the slots by expert and run each expert as one matrix product.  Below it the
     # per-token kernels above are used: no host synchronisation, a fixed launch sequence.
@@ -410,42 +505,48 @@ class HipOps:
     moe_token_slots = 8
     moe_expert_major_slots = 1024
 
-    def _moe_experts_expert_major(self, h, up, down, idx, wt, a=1):
+    def _combine(self, h, ys, inv, idx, wt, E):
+        """y[t] = sum_k wt[t, k] * (ys[inv[t K + k]], or h[t] where idx[t, k] names an identity expert)."""
+        T, D = h.shape
+        y = torch.empty((T, D), dtype=self.dtype, device=h.device)
+        self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, idx.size(1), D, idx.data_ptr(),
+                                          h.data_ptr(), E, self.code, self._s()), "moe_combine")
+        return y
+
+    def _moe_experts_expert_major(self, h, up, down, idx, wt, a=1, limit=0.0):
         T, D = h.shape
         E, rows, K = up.size(0), up.size(1), idx.size(1)
-        ff = rows // 2 if a == 2 else rows
+        ff = rows // 2 if a >= 2 else rows
         n = T * K
         expert, order = torch.sort(idx.reshape(-1).long(), stable=True)   # order: sorted slot -> slot (t K + k)
-        # first sorted slot of every expert (and the end): a search in the sorted list - no count has to reach the host
+        # first sorted slot of every expert (and the end): a search in the sorted list - no count has to reach the host.  Slots of
+        # identity experts (indices from E on) sort behind the last offset and are left to the combine.
         offsets = torch.searchsorted(expert, torch.arange(E + 1, device=h.device))
         inv = torch.empty_like(order)
         inv[order] = torch.arange(n, device=h.device)                  # slot -> sorted slot
         act = torch.empty((n, ff), dtype=self.dtype, device=h.device)
         ys = torch.empty((n, D), dtype=self.dtype, device=h.device)
         self.check(self.L.qsv_expert_rows(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), offsets.data_ptr(),
-                                          E, rows, D, a, self._s()), "expert_rows(up)")
-        self.check(self.L.qsv_expert_rows(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), offsets.data_ptr(), E, D, ff, 0,
+                                          E, rows, D, a, float(limit), self._s()), "expert_rows(up)")
+        self.check(self.L.qsv_expert_rows(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), offsets.data_ptr(), E, D, ff, 0, 0.0,
                                           self._s()), "expert_rows(down)")
-        y = torch.empty((T, D), dtype=self.dtype, device=h.device)
-        self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, K, D, self.code,
-                                          self._s()), "moe_combine")
-        return y
+        return self._combine(h, ys, inv, idx, wt, E)
 
-    def _moe_experts_sorted(self, h, up, down, idx, wt, code=1):
-        """code = 2 (gated units): the grouped kernel folds the two halves of a unit in its epilogue; with vendor products the
+    def _moe_experts_sorted(self, h, up, down, idx, wt, code=1, limit=0.0):
+        """code >= 2 (gated units): the grouped kernel folds the two halves of a unit in its epilogue; with vendor products the
         first product leaves both halves ([n, 2 ff]) and `glu` folds them."""
         T, D = h.shape
         E, rows, K = up.size(0), up.size(1), idx.size(1)
-        ff = rows // 2 if code == 2 else rows
+        ff = rows // 2 if code >= 2 else rows
         n = T * K
         flat = idx.reshape(-1)
         order = torch.argsort(flat, stable=True)                       # sorted slot -> slot (t K + k)
-        counts = torch.bincount(flat, minlength=E).tolist()            # (host synchronisation: the runs' lengths)
+        counts = torch.bincount(flat, minlength=E).tolist()[:E]        # (host synchronisation: the runs' lengths; identity experts sort last)
         inv = torch.empty_like(order)
         inv[order] = torch.arange(n, device=h.device)                  # slot -> sorted slot
         ks, ts = self.L.qsv_grouped_gemm_k_step(), self.L.qsv_grouped_gemm_tile_slots()
         if self.moe_grouped_kernel and self.code == BF16 and D % ks == 0 and ff % ks == 0:
-            # own grouped matrix-core kernel: gather in its loads, relu^2 in the first product's epilogue
+            # own grouped matrix-core kernel: gather in its loads, the activation in the first product's epilogue
             tiles, a = [], 0
             for e, c in enumerate(counts):
                 tiles += [(e, a + o, min(ts, c - o)) for o in range(0, c, ts)]
@@ -455,13 +556,10 @@ class HipOps:
             for lo in range(0, len(tiles), 65535):
                 tl = torch.tensor(tiles[lo:lo + 65535], dtype=torch.int32).to(h.device)
                 self.check(self.L.qsv_grouped_gemm(act.data_ptr(), h.data_ptr(), order.data_ptr(), K, up.data_ptr(), tl.data_ptr(),
-                                                   tl.size(0), rows, D, code, self._s()), "grouped_gemm(up)")
+                                                   tl.size(0), rows, D, code, float(limit), self._s()), "grouped_gemm(up)")
                 self.check(self.L.qsv_grouped_gemm(ys.data_ptr(), act.data_ptr(), 0, 1, down.data_ptr(), tl.data_ptr(),
-                                                   tl.size(0), D, ff, 0, self._s()), "grouped_gemm(down)")
-            y = torch.empty((T, D), dtype=self.dtype, device=h.device)
-            self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, K, D, self.code,
-                                              self._s()), "moe_combine")
-            return y
+                                                   tl.size(0), D, ff, 0, 0.0, self._s()), "grouped_gemm(down)")
+            return self._combine(h, ys, inv, idx, wt, E)
         xs = torch.empty((n, D), dtype=self.dtype, device=h.device)
         self.check(self.L.qsv_gather_rows(xs.data_ptr(), h.data_ptr(), order.data_ptr(), K, n, D, self.code, self._s()),
                    "gather_rows")
@@ -472,8 +570,8 @@ class HipOps:
             if c:
                 torch.matmul(xs[at:at + c], up[e].t(), out=act[at:at + c])
             at += c
-        if code == 2:
-            act = self.glu(act)
+        if code >= 2:
+            act = self.glu(act, "silu" if code == 2 else "clamped", limit)
         else:
             self.check(self.L.qsv_relu_sq(act.data_ptr(), act.numel(), self.code, self._s()), "relu_sq")
         at = 0
@@ -481,10 +579,7 @@ class HipOps:
             if c:
                 torch.matmul(act[at:at + c], down[e].t(), out=ys[at:at + c])
             at += c
-        y = torch.empty((T, D), dtype=self.dtype, device=h.device)
-        self.check(self.L.qsv_moe_combine(y.data_ptr(), ys.data_ptr(), inv.data_ptr(), wt.data_ptr(), T, K, D, self.code,
-                                          self._s()), "moe_combine")
-        return y
+        return self._combine(h, ys, inv, idx, wt, E)
 
 
 def _rotate(v, rope, pos, rot_n):
@@ -545,26 +640,40 @@ class TorchOps:
         qr = _rotate(q.view(T, heads, dim + rot_dim)[..., dim:].float(), rope, pos, rot_n)
         return (torch.cat([q_abs.transpose(0, 1).float(), qr], dim=-1) * scale).contiguous()
 
-    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0, chunk=None, bias=None):
+    def latent_attention(self, qf, pool, batch, window, rank, page, variant=0, key_splits=None, q_first=0, chunk=None, bias=None,
+                         keep_first=0, sink=None, pooled=None, pool_block=0):
         T, H, R = qf.shape
         block_table, seq, pos = batch.block_table, batch.seq, batch.pos
         out = torch.empty((T, H, rank), dtype=self.dtype, device=qf.device)
         bt = block_table.long()
         pools = [pool] if pool.dim() == 2 else list(pool)
+        extra = None if pooled is None else ([pooled] if pooled.dim() == 2 else list(pooled))
         per = H // len(pools)
+        per_page = (page + pool_block - 1) // pool_block if pooled is not None else 0
         for t in range(T):
             p = int(pos[t])
             lo = max(0, p - window + 1) if window else 0
             if chunk:
                 lo = max(lo, p - p % chunk)
             j = torch.arange(lo, p + 1, device=qf.device)
+            if keep_first:
+                j = torch.cat([torch.arange(0, min(int(keep_first), lo), device=qf.device), j])
             at = bt[int(seq[t]), j // page] * page + j % page
             for g, pl in enumerate(pools):
+                hs = slice(g * per, (g + 1) * per)
                 rows = pl[at].float()                                                # [n, R]
-                s = qf[t, g * per:(g + 1) * per] @ rows.t()                          # [per, n]
+                s = qf[t, hs] @ rows.t()                                             # [per, n]
                 if bias is not None:
-                    s = s + bias[g * per:(g + 1) * per][:, (p - j).clamp(max=bias.size(1) - 1)]
-                out[t, g * per:(g + 1) * per] = (torch.softmax(s, dim=-1) @ rows[:, :rank]).to(self.dtype)
+                    s = s + bias[hs][:, (p - j).clamp(max=bias.size(1) - 1)]
+                if extra is not None:                                                # blocks wholly before the window
+                    first = torch.arange(max(0, p - window + 1) // pool_block, device=qf.device) * pool_block
+                    more = extra[g][bt[int(seq[t]), first // page] * per_page + (first % page) // pool_block].float()
+                    s, rows = torch.cat([qf[t, hs] @ more.t(), s], dim=-1), torch.cat([more, rows])
+                if sink is not None:
+                    pr = torch.softmax(torch.cat([s, sink[hs, None]], dim=-1), dim=-1)[:, :-1]
+                else:
+                    pr = torch.softmax(s, dim=-1)
+                out[t, hs] = (pr @ rows[:, :rank]).to(self.dtype)
         return out
 
     def sigmoid_gate(self, o, g):
@@ -621,6 +730,55 @@ class TorchOps:
         o.copy_(self._rotate_halves(o.float(), rope, pos, o.size(-1), sign).to(self.dtype))
         return o
 
+
+    # ---- sandwich norms, sink / kept-first / pooled-block attention, element-wise gated recurrence -----------------------------------
+    def add_normed_rms_norm(self, x, y, w_post, w_next, eps):
+        if y is not None:
+            x += self._rms(y, w_post, eps)
+        return None if w_next is None else self._rms(x, w_next, eps).to(self.dtype)
+
+    def relu_sq(self, a):
+        a.copy_((torch.relu(a.float()) ** 2).to(a.dtype))
+        return a
+
+    def qk_norm_rope_prep(self, q, k, v, heads, kv_heads, dim, vdim, q_w, k_w, per_head, eps, rope, rot_n, scale, pool, batch):
+        T = q.size(0)
+
+        def prep(u, w, n):
+            u = self._rms(u.reshape(T, n, dim), w, eps) if per_head else self._rms(u, w, eps).view(T, n, dim)
+            return u if rope is None else _rotate(u, rope, batch.pos, rot_n)
+
+        if k is not None:
+            rows = torch.cat([v.float().reshape(T, kv_heads, vdim), prep(k, k_w, kv_heads)], dim=-1)
+            pool[:, batch.slot] = rows.transpose(0, 1).to(self.dtype)
+        return torch.cat([torch.zeros(T, heads, vdim, device=q.device), prep(q, q_w, heads) * scale], dim=-1).contiguous()
+
+    def pool_blocks(self, pool, pooled, batch, block, page):
+        per_page = (page + block - 1) // block
+        bt = batch.block_table.long()
+        for t in range(batch.n_tokens):
+            p, s = int(batch.pos[t]), int(batch.seq[t])
+            if (p + 1) % block:
+                continue
+            j = torch.arange(p + 1 - block, p + 1, device=pool.device)
+            first = p + 1 - block
+            dst = bt[s, first // page] * per_page + (first % page) // block
+            pooled[:, dst] = (pool[:, bt[s, j // page] * page + j % page].float().sum(1) / block).to(self.dtype)
+
+    def min_gru_scan(self, proj, z_off, x_off, g_off, b_z, b_x, state, batch, width):
+        z = torch.sigmoid(proj[:, z_off:z_off + width].float() + b_z.float())
+        u = proj[:, x_off:x_off + width].float() + b_x.float()
+        c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+        g = proj[:, g_off:g_off + width].float()
+        out = torch.empty_like(z)
+        for slot, first, cnt in batch.items:
+            S = state[slot].clone() if int(batch.pos[first]) else torch.zeros_like(state[slot])
+            for t in range(first, first + cnt):
+                S = (1.0 - z[t]) * S + z[t] * c[t]
+                out[t] = S
+            state[slot] = S
+        return (out * g * torch.sigmoid(g)).to(self.dtype)
+
     # ---- recurrences ----------------------------------------------------------------------------------------------------------
     def decay(self, z, bias, a_log, tau, heads, dim):
         z = z.float() + bias.float()
@@ -629,7 +787,7 @@ class TorchOps:
         rate = torch.exp(a_log.float()).repeat_interleave(dim)
         return torch.exp(-rate * torch.nn.functional.softplus(z)).contiguous()
 
-    def conv_silu_unit(self, proj, off, conv_w, hist, batch, n_unit, unit_dim):
+    def conv_silu_unit(self, proj, off, conv_w, hist, batch, n_unit, unit_dim, act="silu"):
         C, taps = conv_w.shape
         xin = proj[:, off:off + C].to(self.dtype).float()
         out = torch.empty_like(xin)
@@ -639,9 +797,11 @@ class TorchOps:
             past = hist[rd][:taps - 1] if rd >= 0 else torch.zeros((taps - 1, C), device=xin.device)
             seq = torch.cat([past, xin[first:first + cnt]])
             y = sum(seq[j:j + cnt] * w[:, j] for j in range(taps))
-            out[first:first + cnt] = y * torch.sigmoid(y)
+            out[first:first + cnt] = y * torch.sigmoid(y) if act == "silu" else y
             if taps > 1:
                 hist[wr] = seq[cnt:]
+        if not n_unit:
+            return out
         u = out[:, :n_unit * unit_dim].view(-1, n_unit, unit_dim)
         out[:, :n_unit * unit_dim] = (u / torch.sqrt((u * u).sum(-1, keepdim=True) + 1e-6)).view(-1, n_unit * unit_dim)
         return out
@@ -689,9 +849,12 @@ class TorchOps:
     def rms_pair_mean(self, a, wa, b, wb, eps):
         return (0.5 * (self._rms(a, wa, eps) + self._rms(b, wb, eps))).to(self.dtype)
 
-    def glu(self, a, act="silu"):
+    def glu(self, a, act="silu", limit=0.0):
         a = a.float()
         g, u = a[..., 0::2], a[..., 1::2]
+        if act == "clamped":
+            g, u = g.clamp(max=limit), u.clamp(-limit, limit)
+            return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(self.dtype)
         ag = g * torch.sigmoid(g) if act == "silu" else torch.nn.functional.gelu(g, approximate="tanh")
         return (ag * u).to(self.dtype)
 
@@ -758,15 +921,22 @@ class TorchOps:
             m_state[slot] = prev
         return a, b, m
 
-    def moe_experts(self, h, up, down, idx, wt, act="relu_sq"):
+    def moe_experts(self, h, up, down, idx, wt, act="relu_sq", limit=0.0):
         T, D = h.shape
+        E = up.size(0)
         y = torch.zeros((T, D), dtype=torch.float32, device=h.device)
         for k in range(idx.size(1)):
             e = idx[:, k].long()
+            real = e < E
+            e = e.clamp(max=E - 1)
             a = torch.einsum("tfd,td->tf", up[e].float(), h.float())
-            a = torch.relu(a) ** 2 if act == "relu_sq" else self.glu(a.to(self.dtype)).float()
+            if act == "relu_sq":
+                a = torch.relu(a) ** 2
+            else:
+                a = self.glu(a.to(self.dtype), "silu" if act == "swiglu" else "clamped", limit).float()
             a = a.to(self.dtype).float()
-            y += wt[:, k, None] * torch.einsum("tdf,tf->td", down[e].float(), a)
+            o = torch.einsum("tdf,tf->td", down[e].float(), a)
+            y += wt[:, k, None] * torch.where(real[:, None], o, h.float())
         return y.to(self.dtype)
 
 

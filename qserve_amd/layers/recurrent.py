@@ -127,3 +127,24 @@ class MatrixLSTM:
         o = ops.recurrent_scan(proj[:, :o_k], proj[:, o_k:o_v], proj[:, o_v:o_g], a, None, states[0], batch, H, H, d, self.cols,
                                d ** -0.5, kscale=b, v_cols=dv)
         return linear(ops.head_rms_gate(o, self.norm, proj[:, o_g:o_i], "sigmoid", self.eps, vdim=dv, den_m=m), self.w_o)
+
+
+class MinGRU:
+    """A gated recurrence whose gates read only the current token (minGRU): element by element S <- (1 - z) S + z c with the
+    gate z = sigmoid(W_z h + b_z) and the candidate c = u + 1/2 where u = W_x h + b_x >= 0, sigmoid(u) below; the output is
+    W_o (S * silu(W_g h)).  State per sequence: S, float [width], from zero."""
+
+    def __init__(self, ops, *, width, weights):
+        """weights: z, x, g [width, D], z_b, x_b [width], o [D, width]."""
+        self.ops, self.width = ops, int(width)
+        w = weights
+        D = w["z"].size(1)
+        _check(w, {"z": (width, D), "x": (width, D), "g": (width, D), "z_b": (width,), "x_b": (width,), "o": (D, width)}, "minGRU")
+        self.w_in = torch.cat([w["z"], w["x"], w["g"]], dim=0).contiguous()
+        self.b_z, self.b_x, self.w_o = w["z_b"].contiguous(), w["x_b"].contiguous(), w["o"].contiguous()
+        self.cache_rows, self.state_specs = [], [StateSpec((self.width,))]
+
+    def __call__(self, h, batch, pools, states, carry=None):
+        n = self.width
+        proj = linear(h, self.w_in)
+        return linear(self.ops.min_gru_scan(proj, 0, n, 2 * n, self.b_z, self.b_x, states[0], batch, n), self.w_o)

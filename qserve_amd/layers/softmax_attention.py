@@ -119,3 +119,85 @@ class NormedChunkAttention:
                                        v_first, self.mix or 0.0, pool, batch)
         o = ops.latent_attention(qf, pool, batch, None, self.vdim, self.page, q_first=self.vdim, chunk=self.chunk, bias=self.bias)
         return linear(o.view(T, H * self.vdim), self.w_o)
+
+
+class SinkWindowAttention:
+    """Grouped-query attention over a sliding window whose softmax has a sink: a learned number per head joins the denominator,
+    sum_j e^(s_j) + e^(sink_h), and carries no value.  score = q . k * scale.  Options, all parameters:
+
+    * norm "head": q and k are RMS-normed per head with one weight [dim] shared by the heads; "all": over the whole projection
+      with a weight as wide as it.
+    * taps: a short causal convolution over time on every channel of q, k and v (weights [channels, taps], no bias, no
+      activation) straight after the projection; the last taps - 1 projected rows of a sequence are its state (two copies).
+    * rotary (a RotaryTable): the first rotary.dims dimensions of every q and k head turn with the position, neighbours paired.
+    * keep_first: the first that many positions stay visible to every later query, at their true positions.
+    * pool_block = P: beside the window's tokens a query at i sees one key and one value per block [bP, bP + P) that ends at or
+      before i - window: the means of the block's cached keys and values (a second pool, ceil(page / P) rows per page).
+    * shared_kv: the layer has no keys and values of its own and reads the pools of another layer of the same head counts.
+    Cache: per key / value head one pool of rows [v | k] (k after norm and rotation), as the row-attention kernels read them."""
+
+    def __init__(self, ops, *, heads, kv_heads, dim, vdim, scale, eps, window, weights, norm="head", taps=None, rotary=None,
+                 keep_first=0, pool_block=None, shared_kv=False, page=64):
+        """weights: q [H dim, D], o [D, H vdim], q_norm, sink [H]; unless shared_kv: k [G dim, D], v [G vdim, D], k_norm; with
+        taps: q_conv [H dim, taps], k_conv, v_conv."""
+        if heads % kv_heads or norm not in ("head", "all") or not window or int(window) < 1:
+            raise ValueError(f"attention: {heads} heads over {kv_heads}, norm {norm!r}, window {window}")
+        if shared_kv and (taps or pool_block):
+            raise ValueError("attention: a layer that reads another layer's keys and values has no convolution or pooled blocks")
+        if pool_block and keep_first:
+            raise ValueError("attention: pooled blocks and kept first tokens are alternatives")
+        if pool_block and not 0 < int(pool_block) <= page * 64:
+            raise ValueError(f"attention: pooled blocks of {pool_block} positions")
+        self.ops, self.H, self.G, self.dim, self.vdim, self.page = ops, heads, kv_heads, dim, vdim, page
+        self.scale, self.eps, self.window, self.keep_first = float(scale), float(eps), int(window), int(keep_first or 0)
+        self.per_head, self.taps, self.rotary, self.shared_kv = norm == "head", int(taps) if taps else None, rotary, bool(shared_kv)
+        self.pool_block = int(pool_block) if pool_block else None
+        if rotary is not None and rotary.dims > dim:
+            raise ValueError(f"attention: {rotary.dims} rotated dimensions in heads of {dim}")
+        w = weights
+        D = w["q"].size(1)
+        expect = {"q": (heads * dim, D), "o": (D, heads * vdim), "sink": (heads,), "q_norm": (dim if self.per_head else heads * dim,)}
+        if not shared_kv:
+            expect.update(k=(kv_heads * dim, D), v=(kv_heads * vdim, D), k_norm=(dim if self.per_head else kv_heads * dim,))
+        if self.taps:
+            expect.update(q_conv=(heads * dim, self.taps), k_conv=(kv_heads * dim, self.taps), v_conv=(kv_heads * vdim, self.taps))
+        for k, shp in expect.items():
+            if tuple(w[k].shape) != shp:
+                raise ValueError(f"attention weight {k}: shape {tuple(w[k].shape)}, expected {shp}")
+        self.w_in = (w["q"] if shared_kv else torch.cat([w["q"], w["k"], w["v"]], dim=0)).contiguous()
+        self.w_o, self.q_norm, self.k_norm = w["o"].contiguous(), w["q_norm"].contiguous(), None if shared_kv else w["k_norm"].contiguous()
+        self.sink = w["sink"].float().contiguous()
+        self.conv = torch.cat([w["q_conv"], w["k_conv"], w["v_conv"]], dim=0).float().contiguous() if self.taps else None
+        self.C = (heads + kv_heads) * dim + kv_heads * vdim
+        R = vdim + dim
+        self.cache_rows, self.state_specs = [], []
+        if not shared_kv:
+            self.cache_rows.append((kv_heads, R))
+            if self.pool_block:
+                if self.pool_block > page:
+                    raise ValueError(f"attention: pooled blocks of {self.pool_block} positions on pages of {page}")
+                self.cache_rows.append((kv_heads, R, (page + self.pool_block - 1) // self.pool_block))
+        if self.taps and self.taps > 1:
+            from ..serving.cache import StateSpec
+            self.state_specs.append(StateSpec((self.taps - 1, self.C), copies=2))
+
+    def __call__(self, h, batch, pools, states, carry=None):
+        ops, T, H, G, d, dv = self.ops, h.size(0), self.H, self.G, self.dim, self.vdim
+        proj = linear(h, self.w_in)
+        if self.taps and self.taps > 1:
+            proj = ops.conv_silu_unit(proj, 0, self.conv, states[0], batch, 0, 1, act="none")          # float [T, C]
+        elif self.taps:
+            proj = proj.float() * self.conv[:, 0]
+        q = proj[:, :H * d]
+        k, v = (None, None) if self.shared_kv else (proj[:, H * d:(H + G) * d], proj[:, (H + G) * d:])
+        rope = self.rotary.reserve(batch.max_pos + 1) if self.rotary is not None else None
+        pool = pools[0]
+        qf = ops.qk_norm_rope_prep(q, k, v, H, G, d, dv, self.q_norm, self.k_norm, self.per_head, self.eps, rope,
+                                   self.rotary.dims if rope is not None else 0, self.scale, pool, batch)
+        pooled = None
+        if self.pool_block:
+            pooled = pools[1]
+            ops.pool_blocks(pool, pooled, batch, self.pool_block, self.page)
+        o = ops.latent_attention(qf, pool, batch, self.window, dv, self.page, q_first=dv, keep_first=self.keep_first, sink=self.sink,
+                                 pooled=pooled, pool_block=self.pool_block or 0)
+        return linear(o.view(T, H * dv), self.w_o)

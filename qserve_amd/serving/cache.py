@@ -2,7 +2,8 @@
 
 One page id space serves every layer: page p is rows [p * page, (p + 1) * page) of each layer's pool, and a pool's rows are as
 wide as that layer's cached state per token (layers may differ; a width (n, w) makes n pools of one allocation, [n, rows, w]:
-the key / value heads of one attention layer).  A live sequence owns a slot (a row of the block table) and the pages its
+the key / value heads of one attention layer; (n, w, r) gives a page r rows instead of `page`: state kept per block of B
+positions with r = ceil(page / B), the block that starts in page p at offset o owning row p r + o // B).  A live sequence owns a slot (a row of the block table) and the pages its
 tokens fill; both go back to the free lists when it ends and are handed out again, most recently freed first.
 
 State that does not grow with the sequence (a recurrent matrix, the last inputs of a short convolution, the previous token of
@@ -34,8 +35,15 @@ class PagedCache:
             raise ValueError("the cache needs at least one page and one slot")
         self.page, self.num_pages, self.max_seqs = page, int(num_pages), int(max_seqs)
         rows = self.num_pages * page
-        self.pools = [torch.zeros((rows, w) if isinstance(w, int) else (int(w[0]), rows, int(w[1])), dtype=dtype, device=device)
-                      for w in row_widths]
+        self.pools = []
+        for w in row_widths:
+            if isinstance(w, int):
+                shape = (rows, w)
+            else:
+                if len(w) > 2 and not 0 < int(w[2]) <= page:
+                    raise ValueError(f"a page of {page} positions cannot hold {w[2]} block rows")
+                shape = (int(w[0]), self.num_pages * int(w[2]) if len(w) > 2 else rows, int(w[1]))
+            self.pools.append(torch.zeros(shape, dtype=dtype, device=device))
         self.states = [torch.zeros((self.max_seqs * s.copies,) + s.shape, dtype=s.dtype, device=device) for s in states]
         self.parity = [0] * self.max_seqs
         self.free_pages = list(range(self.num_pages - 1, -1, -1))      # pop() -> lowest id first; freed pages are reused first

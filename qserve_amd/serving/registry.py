@@ -15,7 +15,8 @@ import json
 import os
 
 _MODELS = {}
-_BUILTIN = ("qserve_amd.models.vekalorn", "qserve_amd.models.mumelix", "qserve_amd.models.vepolix", "qserve_amd.models.llama_w4a8")
+_BUILTIN = ("qserve_amd.models.vekalorn", "qserve_amd.models.mumelix", "qserve_amd.models.vepolix", "qserve_amd.models.pemolorn",
+            "qserve_amd.models.llama_w4a8")
 
 
 def register_model(architecture, engine="paged"):
