@@ -31,6 +31,19 @@ int qsv_embed_sinusoid(float* x, const void* table, const int32_t* tokens, const
  * (h == NULL: the sum only). */
 int qsv_add_rms_norm(float* x, void* h, const void* a, const void* b, const void* c, const void* w, float eps, int n_tokens,
                      int width, int dtype, void* stream);
+/* Sublayers between two norms: x[t] += rms_norm(y[t]) * w_post (y == NULL: nothing added), then h[t] = rms_norm(x[t]) * w_next in
+ * the storage type (h == NULL: the sum only).  A weight is one gain for all coordinates (its *_wide flag 0) or one per coordinate. */
+int qsv_add_normed_rms_norm(float* x, void* h, const void* y, const void* w_post, int post_wide, const void* w_next, int next_wide,
+                            float eps, int n_tokens, int width, int dtype, void* stream);
+/* Queries and keys RMS-normed per head (per_head != 0: weights [dim], shared by the heads) or over the whole projection (weights
+ * [heads * dim] / [kv_heads * dim]), then turned by the position: pair (2i, 2i + 1), i < rot_n / 2, of every head by rope[pos[t], :,
+ * i] (float [positions, 2, rot_n / 2], cos then sin; rope == NULL: no rotation).  q, k, v: rows of type qkv_dtype with their strides.
+ *   qf[t, h]         = [ 0 (vdim) | q'[t, h] * scale ]     float [T, heads, vdim + dim]
+ *   pool[g, slot[t]] = [ v[t, g] | k'[t, g] ]              [kv_heads, pool_rows, vdim + dim]     (k == NULL: nothing is written) */
+int qsv_qk_norm_rope_prep(float* qf, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                          int64_t v_stride, int qkv_dtype, int heads, int kv_heads, int dim, int vdim, const void* q_w,
+                          const void* k_w, int per_head, float eps, const float* rope, int rot_n, float scale, void* pool,
+                          int64_t pool_rows, const int64_t* slot, const int32_t* pos, int n_tokens, int dtype, void* stream);
 /* out[r] = rms_norm(x[rows[r]]) * w in the storage type (rows == NULL: row r). */
 int qsv_rms_norm_rows(void* out, const float* x, const int32_t* rows, const void* w, float eps, int n_rows, int width, int dtype,
                       void* stream);
@@ -75,11 +88,24 @@ int qsv_latent_query(float* qf, const void* q, const void* q_abs, const float* r
  * elements after pool g - 1 (one pool for all heads: heads_per_pool = heads, pool_stride = 0). */
 /* Two further restrictions and one further term, for attention layers that have them (0 / NULL: none):
  *   chunk > 0:  only j with floor(j / chunk) == floor(pos[t] / chunk) are visible (chunks counted from position 0);
- *   bias:       float [heads, bias_len]; bias[h, min(pos[t] - j, bias_len - 1)] is added to the score (after the query's scale). */
+ *   bias:       float [heads, bias_len]; bias[h, min(pos[t] - j, bias_len - 1)] is added to the score (after the query's scale).
+ * Keys behind the window and a sink (0 / NULL: none; both need window > 0 and chunk == 0):
+ *   keep_first: positions j < keep_first stay visible to every later query;
+ *   sink:       float [heads]; exp(sink[h]) is one more term of the softmax's denominator, without a value;
+ *   pooled:     a second set of pools (pooled_stride elements apart, same row layout), block_rows rows per page: the block of
+ *               pool_block positions that starts at position s of the sequence has row block_table[s / page] * block_rows +
+ *               (s % page) / pool_block (written by qsv_pool_blocks).  A query at position p also sees the rows of the blocks
+ *               b < (p - window + 1) / pool_block, those that end before its window starts; no bias with them. */
 int qsv_latent_attention(void* out, const float* qf, const void* pool, const int32_t* block_table, int table_stride,
                          const int32_t* seq, const int32_t* pos, int window, int n_tokens, int heads, int rank,
                          int row_width, int page, int heads_per_pool, int64_t pool_stride, int chunk, const float* bias,
-                         int bias_len, int dtype, int variant, void* stream);
+                         int bias_len, int keep_first, const float* sink, const void* pooled, int64_t pooled_stride, int pool_block,
+                         int block_rows, int dtype, int variant, void* stream);
+/* pooled[g, row(block)] = mean over the block's positions of pool[g, row(position)], for every token of the step whose position
+ * ends a block of pool_block positions ((pos + 1) % pool_block == 0); float sum, one rounding. */
+int qsv_pool_blocks(void* pooled, int64_t pooled_rows, const void* pool, int64_t pool_rows, const int32_t* block_table,
+                    int table_stride, const int32_t* seq, const int32_t* pos, int n_tokens, int n_pools, int row_width,
+                    int pool_block, int page, int block_rows, int dtype, void* stream);
 
 int qsv_latent_attention_tile_tokens(int heads);
 int qsv_latent_attention_mfma_ok(int rank, int row_width, int dtype);
@@ -94,7 +120,8 @@ int qsv_latent_attention_mfma(void* out, const float* qf, const void* pool, cons
                               const int32_t* pos, const int32_t* tiles, int n_tiles, int window, int heads, int rank,
                               int row_width, int page, int key_splits, float* part_o, float* part_ml, int n_tokens,
                               int q_first, int heads_per_pool, int64_t pool_stride, int chunk, const float* bias, int bias_len,
-                              void* stream);
+                              int keep_first, const float* sink, const void* pooled, int64_t pooled_stride, int pool_block,
+                              int block_rows, void* stream);
 
 /* o[t, i] *= sigmoid(g[t * g_stride + i]),  i < n. */
 int qsv_sigmoid_gate(void* o, const void* g, int64_t g_stride, int n_tokens, int n, int dtype, void* stream);
@@ -117,13 +144,17 @@ int qsv_moe_route(int32_t* idx, float* weight, const void* h, const void* router
 #define QSV_ACT_NONE 0
 #define QSV_ACT_RELU_SQ 1
 #define QSV_ACT_GLU 2
+/* QSV_ACT_CLAMPED_GLU: the same pairs with g = min(gate, limit), u = clamp(up, -limit, limit), output f = g sigmoid(1.702 g) (u + 1);
+ * `limit` is read by this activation only.  Expert indices >= n_experts name identity experts (output = input): the up kernels
+ * skip their slots and the down / combine kernels add weight * h[t] for them. */
+#define QSV_ACT_CLAMPED_GLU 3
 /* act[t, k] = activation(up[idx[t, k]] . h[t])     up: [E, ff, width] -> act [T, top_k, ff or ff / 2] (storage type). */
 int qsv_moe_up(void* act, const void* h, const void* up, const int32_t* idx, int n_tokens, int top_k, int width, int ff,
-               int activation, int dtype, void* stream);
+               int activation, float limit, int n_experts, int dtype, void* stream);
 
 /* y[t] = sum_k weight[t, k] * down[idx[t, k]] . act[t, k]     down: [E, width, ff] -> y [T, width] (storage type). */
 int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx, const float* weight, int n_tokens,
-                 int top_k, int width, int ff, int dtype, void* stream);
+                 int top_k, int width, int ff, const void* h, int n_experts, int dtype, void* stream);
 
 /* Expert-sorted form for many tokens: slots (t, k) are sorted by expert on the host side of the ABI, the expert products run
  * as ordinary matrix products over contiguous runs of sorted slots, and these kernels do the rest:
@@ -134,18 +165,19 @@ int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx,
  * s in [offsets[e], offsets[e + 1]) of every expert e; W [n_experts, rows, K]; act = one of QSV_ACT_* (QSV_ACT_GLU: out is
  * rows / 2 wide).  Every weight is read once per launch.  K a multiple of 8, at most 4096. */
 int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int64_t* offsets,
-                    int n_experts, int rows, int K, int act, void* stream);
+                    int n_experts, int rows, int K, int act, float limit, void* stream);
 /* Grouped expert product on the bf16 matrix cores (prompt phase): the same out[s, n] for work tiles (expert, first sorted slot,
  * slots <= qsv_grouped_gemm_tile_slots()) listed in tiles int32 [n_tiles, 3]; K a multiple of qsv_grouped_gemm_k_step(), n_rows
  * a multiple of 4, n_tiles <= 65535.  act: QSV_ACT_* (QSV_ACT_GLU: out is n_rows / 2 wide). */
 int qsv_grouped_gemm_tile_slots(void);
 int qsv_grouped_gemm_k_step(void);
 int qsv_grouped_gemm(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int32_t* tiles,
-                     int n_tiles, int n_rows, int K, int act, void* stream);
+                     int n_tiles, int n_rows, int K, int act, float limit, void* stream);
 int qsv_gather_rows(void* out, const void* src, const int64_t* order, int div, int n_rows, int width, int dtype, void* stream);
 int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream);
+/* (idx != NULL: slots with idx[t, k] >= n_experts take h[t] in place of a sorted row) */
 int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n_tokens, int top_k, int width,
-                    int dtype, void* stream);
+                    const int32_t* idx, const void* h, int n_experts, int dtype, void* stream);
 
 
 /* ---- several residual streams, statistics-free norm, token shift (serve_streams.hip) ---------------------------------------- */
@@ -171,20 +203,21 @@ int qsv_rms_pair_mean(void* out, const void* a, const void* wa, const void* b, c
 /* out[r, f] = act(a[r, 2f]) * a[r, 2f + 1]     a: [n_rows, 2 ff]; act QSV_GLU_SILU or QSV_GLU_GELU_TANH (gelu in its tanh form) */
 #define QSV_GLU_SILU 0
 #define QSV_GLU_GELU_TANH 1
-int qsv_glu(void* out, const void* a, int n_rows, int ff, int act, int dtype, void* stream);
+#define QSV_GLU_CLAMPED 2   /* g = min(gate, limit), u = clamp(up, -limit, limit): g sigmoid(1.702 g) (u + 1) */
+int qsv_glu(void* out, const void* a, int n_rows, int ff, int act, float limit, int dtype, void* stream);
 
 /* ---- matrix-state recurrences and the attention beside them (serve_recurrent.hip) ------------------------------------------- */
 /* out[t, c] (float, [T, heads * dim]) = a_log ? exp(-exp(a_log[c / dim]) * softplus(z[t, c] + bias[c]))
  *                                             : sigmoid(z[t, c] + bias[c]) ^ (1 / tau) */
 int qsv_decay(float* out, const void* z, int64_t z_stride, const void* bias, const float* a_log, float tau, int n_tokens,
               int heads, int dim, int dtype, void* stream);
-/* Causal convolution over time per channel, then silu, of the columns [off, off + channels) of proj; w float [channels, taps],
+/* Causal convolution over time per channel, then silu (act 1; act 0: no activation), of the columns [off, off + channels) of proj; w float [channels, taps],
  * the last tap is the current token's.  Inputs before a run's start come from hist[state_rd[t]] (float [2 * slots, taps - 1,
  * channels], oldest first; zeros if state_rd[t] < 0); the run's last token (state_wr[t] >= 0) writes the new history.  The
  * first n_unit groups of unit_dim channels are then divided by sqrt(sum of squares + 1e-6).  out: float [T, channels]. */
 int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, int channels, int taps, const float* w,
                        float* hist, const int32_t* run_off, const int32_t* state_rd, const int32_t* state_wr, int n_unit,
-                       int unit_dim, int n_tokens, int dtype, void* stream);
+                       int unit_dim, int act, int n_tokens, int dtype, void* stream);
 /* Per run (slot, first token, tokens, first position) and head, token by token, with S = state[slot, head] (float [dim, vdim],
  * zeros if the first position is 0) written back at the end, g = decay[t, head]:
  *   beta == NULL:  S <- diag(g) S + k v^T                                  o = S^T q * q_scale
@@ -196,6 +229,11 @@ int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, in
  * kscale (float [T, heads]): k is multiplied by kscale[t, head] where it enters the state; v_cols < vdim: v has v_cols columns per
  * head and the state's column v_cols is fed with ones (it then holds sum of decayed kscale k: a normaliser, read out by q like
  * the others), further columns with zeros. */
+/* Element-wise gated recurrence over every run (slot, first token, tokens, first position): S = state[slot] (float [width], zeros
+ * if the first position is 0), per token S <- (1 - z) S + z c with z = sigmoid(proj[t, z_off + i] + b_z[i]), u = proj[t, x_off + i] +
+ * b_x[i], c = u + 1/2 if u >= 0 else sigmoid(u); out[t, i] = S * silu(proj[t, g_off + i]) (storage type); S is written back. */
+int qsv_min_gru_scan(void* out, const void* proj, int64_t stride, int z_off, int x_off, int g_off, const void* b_z, const void* b_x,
+                     float* state, const int32_t* runs, int n_runs, int width, int dtype, void* stream);
 int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                        int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
                        int beta_dtype, float* state, const int32_t* runs, int n_runs, int max_run, int heads, int qk_heads,

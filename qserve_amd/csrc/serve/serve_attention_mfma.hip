@@ -11,6 +11,12 @@
 // A tile with few tokens (decoding: one) does not fill four waves with rows; then the waves split the KEY tiles among them and
 // merge their partial softmax results through LDS at the end.
 // Scores, running maxima and sums are float; q and the probabilities enter the matrix cores as bfloat16.
+//
+// Keys behind the window: a workgroup's key tiles are numbered, first nA tiles of such keys, then the tiles from the window's start.
+// With `keep_first` these are the tiles of the sequence's first positions that lie wholly below the window's first tile (a kept
+// position inside a window tile is simply visible there); with `pooled` they are tiles of 32 consecutive BLOCKS, one row per block of
+// `pool_block` positions from a second pool, each row addressed through the page of the block's first position.  A sink starts the
+// softmax state of the rows' first key split at (maximum = sink, sum = 1).
 #include "serve_common.h"
 
 namespace {
@@ -31,7 +37,9 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     bf16_t* __restrict__ out, const float* __restrict__ qf, const bf16_t* __restrict__ pool_base,
     const int32_t* __restrict__ block_table, int table_stride, const int32_t* __restrict__ pos, const int32_t* __restrict__ tiles,
     int window, int H, int rank, int R, int page, int HP, int TQ, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int n_tokens, int s_lo, int s_hi, int per, int64_t pool_stride, int chunk, const float* __restrict__ bias, int bias_len) {
+    int n_tokens, int s_lo, int s_hi, int per, int64_t pool_stride, int chunk, const float* __restrict__ bias, int bias_len,
+    int keep_first, const float* __restrict__ sink, const bf16_t* __restrict__ pooled_base, int64_t pooled_stride, int pool_block,
+    int block_rows) {
     constexpr int RS = 32 * RT + 8;                      // row stride (elements) of the row-major tile
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     bf16_t* Ks = (bf16_t*)smem;                          // [BN][RS]
@@ -45,6 +53,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     const int gpp = (per + 15) / 16, pool_id = blockIdx.y / gpp;
     const int h0 = pool_id * per + (blockIdx.y % gpp) * 16, h_end = pool_id * per + per;
     const bf16_t* __restrict__ pool = pool_base + (size_t)pool_id * (size_t)pool_stride;
+    const bf16_t* __restrict__ pooled = pooled_base ? pooled_base + (size_t)pool_id * (size_t)pooled_stride : nullptr;
     const int32_t* bt = block_table + (size_t)slot * table_stride;
 
     // rows of this wave: group grp of TQ tokens, key split sp
@@ -66,6 +75,11 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     int lo_first = window > 0 ? max(0, p_first - window + 1) : 0;
     if (chunk > 0) lo_first = max(lo_first, p_first - p_first % chunk);   // (the first token's bound is the tile's lowest)
     const int kstart = (lo_first / BN) * BN;
+    // tiles of keys behind the window, and each row's count of such keys
+    const int nb_last = pooled ? max(0, p_last - window + 1) / pool_block : 0;      // blocks the tile's last token sees
+    const int nb_row = pooled ? max(0, p_row - window + 1) / pool_block : 0;
+    const int nA = pooled ? (nb_last + BN - 1) / BN : (keep_first > 0 ? min((keep_first + BN - 1) / BN, kstart / BN) : 0);
+    const int nT = nA + (p_last - kstart) / BN + 1;
     // wave key range: rows of this wave's group
     const int gt_first = min(grp * TQ, ntok - 1), gt_last = min(grp * TQ + TQ - 1, ntok - 1);
     const int wp_last = p_first + gt_last;
@@ -91,6 +105,10 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
 #pragma unroll
     for (int c = 0; c < CT; ++c) oacc[c] = v4f{0.f, 0.f, 0.f, 0.f};
     float m = -INFINITY, l = 0.f;
+    if (sink && row_ok && sp == 0 && blockIdx.z == 0) {  // the sink's term: once per row, in its first key split
+        m = sink[head];
+        l = g4 == 0 ? 1.f : 0.f;                         // (l is a lane's share of the row's sum)
+    }
 
     const int chunks_per_row = R / 8;                    // 16-byte pieces of a cache row (R % 8 == 0)
     // gridDim.z > 1 (decoding with few sequences): workgroup z takes every gridDim.z-th key tile and leaves an unnormalised
@@ -100,7 +118,21 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
     // pieces of the NEXT tile are in flight (registers) while this tile is computed from LDS.
     constexpr int NCH = (BN * 4 * RT + 64 * NWV - 1) / (64 * NWV);
     v4u stage[NCH];
-    auto issue = [&](int k0) {
+    auto issue = [&](int tile) {
+        if (pooled && tile < nA) {                       // 32 blocks: every row through the page of its block's first position
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int q = tid + 64 * NWV * i, row = q % BN, cc = q / BN;
+                stage[i] = v4u{0u, 0u, 0u, 0u};
+                const int b = tile * BN + row;
+                if (b < nb_last && cc < chunks_per_row) {
+                    const int first = b * pool_block;
+                    stage[i] = *(const v4u*)(pooled + ((size_t)bt[first / page] * block_rows + (size_t)((first % page) / pool_block)) * (size_t)R + cc * 8);
+                }
+            }
+            return;
+        }
+        const int k0 = tile < nA ? tile * BN : kstart + (tile - nA) * BN;
         const bf16_t* base = pool + ((size_t)bt[k0 / page] * page + (size_t)(k0 % page)) * (size_t)R;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
@@ -110,9 +142,10 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
         }
     };
     int ti = 0;
-    const int kfirst = kstart + z * BN;
-    if (kfirst <= p_last) issue(kfirst);
-    for (int k0 = kfirst; k0 <= p_last; k0 += Z * BN, ++ti) {
+    if (z < nT) issue(z);
+    for (int tile = z; tile < nT; tile += Z, ++ti) {
+        const bool pre = tile < nA;                      // (block-uniform) a tile of keys behind the window
+        const int k0 = pre ? tile * BN : kstart + (tile - nA) * BN;
         __syncthreads();                                 // the previous tile has been read
         // ---- the staged rows into LDS: row-major and transposed (lanes walk the rows: the 2-byte transposed writes of a
         //      wave fall into 32 different banks) ----
@@ -132,8 +165,9 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
             }
         }
         __syncthreads();
-        if (k0 + Z * BN <= p_last) issue(k0 + Z * BN);
-        if (!active || (ti % S) != sp || k0 > wp_last || k0 + BN - 1 < wlo) continue;   // (wave-uniform)
+        if (tile + Z < nT) issue(tile + Z);
+        // (wave-uniform; a tile below the wave's window may still hold kept first positions)
+        if (!active || (ti % S) != sp || (!pre && (k0 > wp_last || (k0 + BN - 1 < wlo && k0 >= keep_first)))) continue;
         // the bias of this lane's eight (query, key) pairs: requested before the score product, added after it
         float bv[2][4];
         if (brow) {
@@ -161,7 +195,7 @@ __global__ __launch_bounds__(64 * NWV, (RT > 10 ? 1 : 2)) void latent_attention_
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int key = k0 + 16 * mt + 4 * g4 + r;
-                const bool vis = key <= p_row && key >= lo_row;
+                const bool vis = (pooled && pre) ? key < nb_row : (key <= p_row && (key >= lo_row || key < keep_first));
                 if (brow) sacc[mt][r] += bv[mt][r];
                 sacc[mt][r] = vis ? sacc[mt][r] : -INFINITY;
                 tmax = fmaxf(tmax, sacc[mt][r]);
@@ -319,7 +353,13 @@ extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void*
                                          int table_stride, const int32_t* pos, const int32_t* tiles, int n_tiles, int window,
                                          int H, int rank, int R, int page, int key_splits, float* part_o, float* part_ml,
                                          int n_tokens, int q_first, int heads_per_pool, int64_t pool_stride, int chunk,
-                                         const float* bias, int bias_len, void* stream) {
+                                         const float* bias, int bias_len, int keep_first, const float* sink, const void* pooled,
+                                         int64_t pooled_stride, int pool_block, int block_rows, void* stream) {
+    QSV_REQUIRE(keep_first >= 0 && (!keep_first || (window > 0 && !chunk)),
+                "qsv_latent_attention_mfma: %d kept first positions need a window and no chunks", keep_first);
+    QSV_REQUIRE(!pooled || (window > 0 && !chunk && !bias && !keep_first && pool_block > 0 && block_rows > 0 && pooled_stride >= 0 &&
+                            (int64_t)block_rows * pool_block >= page),
+                "qsv_latent_attention_mfma: pooled blocks of %d positions, %d rows per page of %d", pool_block, block_rows, page);
     QSV_REQUIRE(chunk >= 0 && (!bias || bias_len > 0), "qsv_latent_attention_mfma: chunk %d, bias table of %d distances", chunk, bias_len);
     QSV_REQUIRE(out && qf && pool && block_table && pos && tiles, "qsv_latent_attention_mfma: null argument");
     QSV_REQUIRE(qsv_latent_attention_mfma_ok(rank, R, QSV_BF16) && R >= rank && H > 0 && page > 0 && page % BN == 0 && window >= 0 && n_tiles >= 0,
@@ -346,7 +386,8 @@ extern "C" int qsv_latent_attention_mfma(void* out, const float* qf, const void*
         }                                                                                                                    \
         hipLaunchKernelGGL((latent_attention_mfma_kernel<RT, CT>), grid, block, lds, (hipStream_t)stream, (bf16_t*)out, qf,  \
                            (const bf16_t*)pool, block_table, table_stride, pos, tiles, window, H, rank, R, page, g.HP, g.TQ, \
-                           part_o, part_ml, n_tokens, s_lo, s_hi, heads_per_pool, pool_stride, chunk, bias, bias_len);        \
+                           part_o, part_ml, n_tokens, s_lo, s_hi, heads_per_pool, pool_stride, chunk, bias, bias_len,         \
+                           keep_first, sink, (const bf16_t*)pooled, pooled_stride, pool_block, block_rows);                       \
     } while (0)
     if (rt <= 4 && ct <= 8) QSV_MFMA(4, 8);
     else if (rt <= 6 && ct <= 12) QSV_MFMA(6, 12);

@@ -161,18 +161,27 @@ __global__ __launch_bounds__(NT) void moe_route_kernel(int32_t* __restrict__ idx
 // Activation of the first expert product.  ACT_GLU: the weight rows come in pairs (2f = gate, 2f + 1 = up) and output f is
 // silu(gate) * up, so the output is half as wide as the product.
 constexpr int ACT_NONE = 0, ACT_RELU_SQ = 1, ACT_GLU = 2;
+// (QSV_ACT_CLAMPED_GLU runs the ACT_GLU kernels with limit > 0: g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(1.702 g) (u + 1))
 __device__ __forceinline__ float relu_sq(float d) {
     const float a = fmaxf(d, 0.f);
     return a * a;
 }
-__device__ __forceinline__ float glu(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+__device__ __forceinline__ float glu(float g, float u, float limit) {
+    if (limit > 0.f) {                                       // (uniform over the launch)
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return g / (1.0f + expf(-g)) * u;
+}
 
 // One workgroup per (token, chosen expert): act = relu(up_e . h)^2 (or the gated unit).  Dynamic LDS: D floats.  ff: weight rows.
 template <typename T, int ACT>
 __global__ __launch_bounds__(NT) void moe_up_kernel(T* __restrict__ act, const T* __restrict__ h, const T* __restrict__ up,
-                                                    const int32_t* __restrict__ idx, int top_k, int D, int ff) {
+                                                    const int32_t* __restrict__ idx, int top_k, int D, int ff, float limit, int n_experts) {
     extern __shared__ float xs[];
     const size_t slot = blockIdx.x;
+    if (idx[slot] >= n_experts) return;                      // an identity expert: the down kernel adds the input itself
     const size_t t = slot / top_k;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < D; i += NT) xs[i] = ld(h, t * D + i);
@@ -188,7 +197,7 @@ __global__ __launch_bounds__(NT) void moe_up_kernel(T* __restrict__ act, const T
             }
             d = wave_sum(d);
             e = wave_sum(e);
-            if (lane == 0) st(act, slot * (ff / 2) + f, glu(d, e));
+            if (lane == 0) st(act, slot * (ff / 2) + f, glu(d, e, limit));
         }
         return;
     }
@@ -205,7 +214,7 @@ __global__ __launch_bounds__(NT) void moe_up_kernel(T* __restrict__ act, const T
 template <typename T>
 __global__ __launch_bounds__(NT) void moe_down_kernel(T* __restrict__ y, const T* __restrict__ act, const T* __restrict__ down,
                                                       const int32_t* __restrict__ idx, const float* __restrict__ weight,
-                                                      int top_k, int D, int ff) {
+                                                      int top_k, int D, int ff, const T* __restrict__ h, int n_experts) {
     extern __shared__ float as[];
     const size_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -214,6 +223,10 @@ __global__ __launch_bounds__(NT) void moe_down_kernel(T* __restrict__ y, const T
     for (int d = w; d < D; d += NW) {
         float total = 0.f;
         for (int k = 0; k < top_k; ++k) {
+            if (idx[t * top_k + k] >= n_experts) {           // identity expert
+                total += weight[t * top_k + k] * ld(h, t * D + d);
+                continue;
+            }
             const T* r = down + ((size_t)idx[t * top_k + k] * D + d) * ff;
             float v = 0.f;
             for (int i = lane; i < ff; i += 64) v += ld(r, i) * as[k * ff + i];
@@ -229,9 +242,10 @@ constexpr int ROWS = 4;      // output rows a wave works on at once
 
 template <typename T, int ACT>
 __global__ __launch_bounds__(NT) void moe_up_vec_kernel(T* __restrict__ act, const T* __restrict__ h, const T* __restrict__ up,
-                                                        const int32_t* __restrict__ idx, int top_k, int D, int ff) {
+                                                        const int32_t* __restrict__ idx, int top_k, int D, int ff, float limit, int n_experts) {
     extern __shared__ float xs[];
     const size_t slot = blockIdx.x;
+    if (idx[slot] >= n_experts) return;                      // an identity expert: the down kernel adds the input itself
     const size_t t = slot / top_k;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < D; i += NT) xs[i] = ld(h, t * D + i);
@@ -260,7 +274,7 @@ __global__ __launch_bounds__(NT) void moe_up_vec_kernel(T* __restrict__ act, con
             if (ACT == ACT_GLU) {                               // (ROWS and ff are even: a pair never straddles two waves)
 #pragma unroll
                 for (int r = 0; r < ROWS; r += 2)
-                    if (f0 + r < ff) st(act, slot * (ff / 2) + (f0 + r) / 2, glu(d[r], d[r + 1]));
+                    if (f0 + r < ff) st(act, slot * (ff / 2) + (f0 + r) / 2, glu(d[r], d[r + 1], limit));
             } else {
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r)
@@ -273,7 +287,7 @@ __global__ __launch_bounds__(NT) void moe_up_vec_kernel(T* __restrict__ act, con
 template <typename T>
 __global__ __launch_bounds__(NT) void moe_down_vec_kernel(T* __restrict__ y, const T* __restrict__ act, const T* __restrict__ down,
                                                           const int32_t* __restrict__ idx, const float* __restrict__ weight,
-                                                          int top_k, int D, int ff) {
+                                                          int top_k, int D, int ff, const T* __restrict__ h, int n_experts) {
     extern __shared__ float as[];
     const size_t t = blockIdx.x;
     const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
@@ -282,8 +296,16 @@ __global__ __launch_bounds__(NT) void moe_down_vec_kernel(T* __restrict__ y, con
     for (int d0 = w * ROWS; d0 < D; d0 += NW * ROWS) {
         float acc[ROWS] = {0.f, 0.f, 0.f, 0.f};
         for (int k = 0; k < top_k; ++k) {
-            const T* Wk = down + (size_t)idx[t * top_k + k] * D * ff;
             const float wk = weight[t * top_k + k];
+            if (idx[t * top_k + k] >= n_experts) {           // identity expert: lane 0's share carries the input (the rest add zero)
+                if (lane == 0) {
+#pragma unroll
+                    for (int r = 0; r < ROWS; ++r)
+                        if (d0 + r < D) acc[r] += wk * ld(h, t * D + d0 + r);
+                }
+                continue;
+            }
+            const T* Wk = down + (size_t)idx[t * top_k + k] * D * ff;
             float part[ROWS] = {0.f, 0.f, 0.f, 0.f};
             for (int c = lane * 8; c < ff; c += 64 * 8) {
                 float x[8];
@@ -317,7 +339,7 @@ typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
 template <int KI, int ACT>
 __global__ __launch_bounds__(NT) void expert_rows_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
                                                          const int64_t* __restrict__ x_index, int div, const bf16_t* __restrict__ W,
-                                                         const int64_t* __restrict__ offsets, int rows, int K) {
+                                                         const int64_t* __restrict__ offsets, int rows, int K, float limit) {
     const int e = blockIdx.y;
     const int64_t s0 = offsets[e], s1 = offsets[e + 1];
     if (s0 == s1) return;                                                   // nobody chose this expert
@@ -369,7 +391,7 @@ __global__ __launch_bounds__(NT) void expert_rows_kernel(bf16_t* __restrict__ ou
                     if (ACT == ACT_GLU) {
 #pragma unroll
                         for (int r = 0; r < ROWS; r += 2)
-                            if (r0 + r < rows) out[(size_t)(sb + j) * (rows / 2) + (r0 + r) / 2] = f2bf(glu(d[r], d[r + 1]));
+                            if (r0 + r < rows) out[(size_t)(sb + j) * (rows / 2) + (r0 + r) / 2] = f2bf(glu(d[r], d[r + 1], limit));
                     } else {
 #pragma unroll
                         for (int r = 0; r < ROWS; ++r)
@@ -401,11 +423,15 @@ __global__ __launch_bounds__(NT) void relu_sq_kernel(T* __restrict__ a, size_t n
 // y[t] = sum_k weight[t, k] * ys[inv[t top_k + k]]
 template <typename T>
 __global__ __launch_bounds__(NT) void moe_combine_kernel(T* __restrict__ y, const T* __restrict__ ys, const int64_t* __restrict__ inv,
-                                                         const float* __restrict__ weight, int top_k, int D) {
+                                                         const float* __restrict__ weight, int top_k, int D,
+                                                         const int32_t* __restrict__ idx, const T* __restrict__ h, int n_experts) {
     const size_t t = blockIdx.x;
     for (int c = threadIdx.x; c < D; c += NT) {
         float a = 0.f;
-        for (int k = 0; k < top_k; ++k) a += weight[t * top_k + k] * ld(ys, (size_t)inv[t * top_k + k] * D + c);
+        for (int k = 0; k < top_k; ++k) {
+            const bool same = idx && idx[t * top_k + k] >= n_experts;       // an identity expert's slot has no sorted row
+            a += weight[t * top_k + k] * (same ? ld(h, t * D + c) : ld(ys, (size_t)inv[t * top_k + k] * D + c));
+        }
         st(y, t * D + c, a);
     }
 }
@@ -423,9 +449,13 @@ extern "C" int qsv_gather_rows(void* out, const void* src, const int64_t* order,
 // out[s, r] = act(W[e][r, :] . X[x_index ? x_index[s] / div : s, :]) for the sorted slots s in [offsets[e], offsets[e + 1]) of every
 // expert e; W [E, rows, K] bfloat16, act: 0 nothing, 1 relu^2, 2 gated unit (row pairs; out is rows / 2 wide).  K % 8 == 0, K <= 4096.
 extern "C" int qsv_expert_rows(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int64_t* offsets,
-                               int n_experts, int rows, int K, int act, void* stream) {
+                               int n_experts, int rows, int K, int act, float limit, void* stream) {
     QSV_REQUIRE(out && X && W && offsets && n_experts > 0 && rows > 0 && div > 0, "qsv_expert_rows: bad arguments");
-    QSV_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQ || (act == ACT_GLU && rows % 2 == 0), "qsv_expert_rows: activation %d", act);
+    QSV_REQUIRE(act == ACT_NONE || act == ACT_RELU_SQ || ((act == ACT_GLU || act == QSV_ACT_CLAMPED_GLU) && rows % 2 == 0),
+                "qsv_expert_rows: activation %d", act);
+    QSV_REQUIRE(act != QSV_ACT_CLAMPED_GLU || limit > 0.f, "qsv_expert_rows: clamped units need a positive limit");
+    if (act == QSV_ACT_CLAMPED_GLU) act = ACT_GLU;
+    else limit = 0.f;
     QSV_REQUIRE(K > 0 && K % 8 == 0 && K <= 4096, "qsv_expert_rows: inner width %d (a multiple of 8, at most 4096)", K);
     QSV_REQUIRE(n_experts <= 65535, "qsv_expert_rows: too many experts");
     const dim3 grid((rows + NW * ROWS - 1) / (NW * ROWS), n_experts), block(NT);
@@ -433,13 +463,13 @@ extern "C" int qsv_expert_rows(void* out, const void* X, const int64_t* x_index,
     do {                                                                                                                     \
         if (act == ACT_RELU_SQ)                                                                                              \
             hipLaunchKernelGGL((expert_rows_kernel<KI, ACT_RELU_SQ>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out,         \
-                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K);                          \
+                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K, limit);                          \
         else if (act == ACT_GLU)                                                                                             \
             hipLaunchKernelGGL((expert_rows_kernel<KI, ACT_GLU>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out,             \
-                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K);                          \
+                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K, limit);                          \
         else                                                                                                                 \
             hipLaunchKernelGGL((expert_rows_kernel<KI, ACT_NONE>), grid, block, 0, (hipStream_t)stream, (bf16_t*)out,            \
-                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K);                          \
+                               (const bf16_t*)X, x_index, div, (const bf16_t*)W, offsets, rows, K, limit);                          \
     } while (0)
     if (K <= 512) QSV_ER(1);
     else if (K <= 1024) QSV_ER(2);
@@ -457,12 +487,12 @@ extern "C" int qsv_relu_sq(void* a, int64_t n, int dtype, void* stream) {
     return qsv_launch_status("qsv_relu_sq");
 }
 extern "C" int qsv_moe_combine(void* y, const void* ys, const int64_t* inv, const float* weight, int n, int top_k, int D,
-                               int dtype, void* stream) {
-    QSV_REQUIRE(y && ys && inv && weight && n >= 0 && top_k > 0 && D > 0, "qsv_moe_combine: bad arguments");
+                               const int32_t* idx, const void* h, int n_experts, int dtype, void* stream) {
+    QSV_REQUIRE(y && ys && inv && weight && n >= 0 && top_k > 0 && D > 0 && (!idx || h), "qsv_moe_combine: bad arguments");
     if (n == 0) return QSV_OK;
     QSV_DISPATCH(dtype, "qsv_moe_combine",
                  hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, (T*)y, (const T*)ys, inv,
-                                    weight, top_k, D));
+                                    weight, top_k, D, idx, (const T*)h, n_experts));
     return qsv_launch_status("qsv_moe_combine");
 }
 
@@ -484,16 +514,19 @@ extern "C" int qsv_moe_route(int32_t* idx, float* weight, const void* h, const v
 }
 
 extern "C" int qsv_moe_up(void* act, const void* h, const void* up, const int32_t* idx, int n, int top_k, int D, int ff,
-                          int activation, int dtype, void* stream) {
-    QSV_REQUIRE(act && h && up && idx && n >= 0 && top_k > 0 && D > 0 && ff > 0, "qsv_moe_up: bad arguments");
-    QSV_REQUIRE(activation == ACT_RELU_SQ || (activation == ACT_GLU && ff % 2 == 0), "qsv_moe_up: activation %d over %d rows",
-                activation, ff);
+                          int activation, float limit, int n_experts, int dtype, void* stream) {
+    QSV_REQUIRE(act && h && up && idx && n >= 0 && top_k > 0 && D > 0 && ff > 0 && n_experts > 0, "qsv_moe_up: bad arguments");
+    QSV_REQUIRE(activation == ACT_RELU_SQ || ((activation == ACT_GLU || activation == QSV_ACT_CLAMPED_GLU) && ff % 2 == 0),
+                "qsv_moe_up: activation %d over %d rows", activation, ff);
+    QSV_REQUIRE(activation != QSV_ACT_CLAMPED_GLU || limit > 0.f, "qsv_moe_up: clamped units need a positive limit");
+    if (activation == QSV_ACT_CLAMPED_GLU) activation = ACT_GLU;
+    else limit = 0.f;
     QSV_REQUIRE((size_t)D * 4 <= 64 * 1024, "qsv_moe_up: width %d does not fit the workgroup's LDS", D);
     if (n == 0) return QSV_OK;
 #define QSV_UP(KERNEL, ACT)                                                                                                  \
     QSV_DISPATCH(dtype, "qsv_moe_up",                                                                                        \
                  hipLaunchKernelGGL((KERNEL<T, ACT>), dim3(n * top_k), dim3(NT), (size_t)D * 4, (hipStream_t)stream, (T*)act,   \
-                                    (const T*)h, (const T*)up, idx, top_k, D, ff))
+                                    (const T*)h, (const T*)up, idx, top_k, D, ff, limit, n_experts))
     if (D % 8 == 0) {
         if (activation == ACT_GLU) QSV_UP(moe_up_vec_kernel, ACT_GLU);
         else QSV_UP(moe_up_vec_kernel, ACT_RELU_SQ);
@@ -506,17 +539,18 @@ extern "C" int qsv_moe_up(void* act, const void* h, const void* up, const int32_
 }
 
 extern "C" int qsv_moe_down(void* y, const void* act, const void* down, const int32_t* idx, const float* weight, int n,
-                            int top_k, int D, int ff, int dtype, void* stream) {
-    QSV_REQUIRE(y && act && down && idx && weight && n >= 0 && top_k > 0 && D > 0 && ff > 0, "qsv_moe_down: bad arguments");
+                            int top_k, int D, int ff, const void* h, int n_experts, int dtype, void* stream) {
+    QSV_REQUIRE(y && act && down && idx && weight && h && n >= 0 && top_k > 0 && D > 0 && ff > 0 && n_experts > 0,
+                "qsv_moe_down: bad arguments");
     QSV_REQUIRE((size_t)top_k * ff * 4 <= 64 * 1024, "qsv_moe_down: %d x %d activations do not fit the workgroup's LDS", top_k, ff);
     if (n == 0) return QSV_OK;
     if (ff % 8 == 0)
         QSV_DISPATCH(dtype, "qsv_moe_down",
                      hipLaunchKernelGGL(moe_down_vec_kernel<T>, dim3(n), dim3(NT), (size_t)top_k * ff * 4, (hipStream_t)stream, (T*)y,
-                                        (const T*)act, (const T*)down, idx, weight, top_k, D, ff));
+                                        (const T*)act, (const T*)down, idx, weight, top_k, D, ff, (const T*)h, n_experts));
     else
         QSV_DISPATCH(dtype, "qsv_moe_down",
                      hipLaunchKernelGGL(moe_down_kernel<T>, dim3(n), dim3(NT), (size_t)top_k * ff * 4, (hipStream_t)stream, (T*)y,
-                                        (const T*)act, (const T*)down, idx, weight, top_k, D, ff));
+                                        (const T*)act, (const T*)down, idx, weight, top_k, D, ff, (const T*)h, n_experts));
     return qsv_launch_status("qsv_moe_down");
 }

@@ -31,7 +31,7 @@ template <int ACT>
 __global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ X,
                                                            const int64_t* __restrict__ x_index, int div,
                                                            const bf16_t* __restrict__ W, const int32_t* __restrict__ tiles, int N,
-                                                           int K) {
+                                                           int K, float limit) {
     __shared__ __attribute__((aligned(16))) bf16_t As[BNW * LS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BS * LS];
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -111,7 +111,15 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(bf16_t* __restrict
             if (n >= N) continue;                                   // N % 4 == 0: the four rows are inside together
             v4f v = acc[mt][nt];
             if (ACT == 2) {
-                const float u0 = v[0] / (1.0f + expf(-v[0])) * v[1], u1 = v[2] / (1.0f + expf(-v[2])) * v[3];
+                float u0, u1;
+                if (limit > 0.f) {                                  // clamped units: g sigmoid(1.702 g) (u + 1) (uniform over the launch)
+                    const float ga = fminf(v[0], limit), gb = fminf(v[2], limit);
+                    u0 = ga / (1.0f + expf(-1.702f * ga)) * (fminf(fmaxf(v[1], -limit), limit) + 1.0f);
+                    u1 = gb / (1.0f + expf(-1.702f * gb)) * (fminf(fmaxf(v[3], -limit), limit) + 1.0f);
+                } else {
+                    u0 = v[0] / (1.0f + expf(-v[0])) * v[1];
+                    u1 = v[2] / (1.0f + expf(-v[2])) * v[3];
+                }
                 *(unsigned*)(out + (size_t)(s_first + sl) * (N / 2) + n / 2) = pack_bf2(u0, u1);
                 continue;
             }
@@ -134,16 +142,19 @@ __global__ __launch_bounds__(256, 2) void grouped_gemm_kernel(bf16_t* __restrict
 extern "C" int qsv_grouped_gemm_tile_slots(void) { return BS; }
 extern "C" int qsv_grouped_gemm_k_step(void) { return KS; }
 extern "C" int qsv_grouped_gemm(void* out, const void* X, const int64_t* x_index, int div, const void* W, const int32_t* tiles,
-                                int n_tiles, int N, int K, int act, void* stream) {
+                                int n_tiles, int N, int K, int act, float limit, void* stream) {
     QSV_REQUIRE(out && X && W && tiles && div > 0 && n_tiles >= 0, "qsv_grouped_gemm: bad arguments");
     QSV_REQUIRE(N > 0 && N % 4 == 0 && K > 0 && K % KS == 0, "qsv_grouped_gemm: N %d (a multiple of 4), K %d (a multiple of 64)", N, K);
     QSV_REQUIRE(n_tiles <= 65535, "qsv_grouped_gemm: %d tiles (at most 65535 per launch)", n_tiles);
-    QSV_REQUIRE(act == QSV_ACT_NONE || act == QSV_ACT_RELU_SQ || act == QSV_ACT_GLU, "qsv_grouped_gemm: activation %d", act);
+    QSV_REQUIRE(act == QSV_ACT_NONE || act == QSV_ACT_RELU_SQ || act == QSV_ACT_GLU || (act == QSV_ACT_CLAMPED_GLU && limit > 0.f),
+                "qsv_grouped_gemm: activation %d (limit %g)", act, (double)limit);
+    if (act == QSV_ACT_CLAMPED_GLU) act = QSV_ACT_GLU;
+    else limit = 0.f;
     if (n_tiles == 0) return QSV_OK;
     const dim3 grid((N + BNW - 1) / BNW, n_tiles), block(256);
 #define QSV_GG(ACT)                                                                                                          \
     hipLaunchKernelGGL(grouped_gemm_kernel<ACT>, grid, block, 0, (hipStream_t)stream, (bf16_t*)out, (const bf16_t*)X, x_index, div, \
-                       (const bf16_t*)W, tiles, N, K)
+                       (const bf16_t*)W, tiles, N, K, limit)
     if (act == QSV_ACT_RELU_SQ) QSV_GG(1);
     else if (act == QSV_ACT_GLU) QSV_GG(2);
     else QSV_GG(0);

@@ -23,7 +23,7 @@ __global__ __launch_bounds__(NT) void decay_kernel(float* __restrict__ out, cons
     }
 }
 
-// ---- causal convolution over time + silu, unit norm of the leading groups -----------------------------------------------------
+// ---- causal convolution over time + silu (act 0: no activation), unit norm of the leading groups -----------------------------------------------------
 // Workgroup = token.  Tap j (last column = the current token) reads the input taps - 1 - j tokens back: a row of this batch
 // inside the run, the sequence's history state before the run's start, zero before the sequence's start.  The last token of a
 // run writes the new history (the last taps - 1 inputs) into the state's other copy.  Dynamic LDS: C floats.
@@ -32,7 +32,7 @@ __global__ __launch_bounds__(NT) void conv_silu_unit_kernel(float* __restrict__ 
                                                             int off, int C, int taps, const float* __restrict__ w,
                                                             float* __restrict__ hist, const int32_t* __restrict__ run_off,
                                                             const int32_t* __restrict__ state_rd,
-                                                            const int32_t* __restrict__ state_wr, int n_unit, int unit_dim) {
+                                                            const int32_t* __restrict__ state_wr, int n_unit, int unit_dim, int act) {
     extern __shared__ float ys[];
     const size_t t = blockIdx.x;
     const int i = run_off[t], rd = state_rd[t], wr = state_wr[t];
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(NT) void conv_silu_unit_kernel(float* __restrict__ 
             else if (rd >= 0) xv = hist[((size_t)rd * past + (past + i - d)) * C + c];
             acc += w[(size_t)c * taps + j] * xv;
         }
-        ys[c] = acc / (1.0f + expf(-acc));
+        ys[c] = act ? acc / (1.0f + expf(-acc)) : acc;
         if (wr >= 0) {
             for (int jj = 0; jj < past; ++jj) {
                 const int e = i + 1 - past + jj;            // index within the run of the input that becomes history entry jj
@@ -516,17 +516,17 @@ extern "C" int qsv_decay(float* out, const void* z, int64_t z_stride, const void
 
 extern "C" int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, int channels, int taps, const float* w,
                                   float* hist, const int32_t* run_off, const int32_t* state_rd, const int32_t* state_wr,
-                                  int n_unit, int unit_dim, int n_tokens, int dtype, void* stream) {
+                                  int n_unit, int unit_dim, int act, int n_tokens, int dtype, void* stream) {
     QSV_REQUIRE(out && proj && w && hist && run_off && state_rd && state_wr, "qsv_conv_silu_unit: null argument");
     QSV_REQUIRE(channels > 0 && taps >= 1 && off >= 0 && off + channels <= stride && n_unit >= 0 && unit_dim > 0 &&
-                    (int64_t)n_unit * unit_dim <= channels && n_tokens >= 0,
+                    (int64_t)n_unit * unit_dim <= channels && n_tokens >= 0 && (act == 0 || act == 1),
                 "qsv_conv_silu_unit: bad sizes");
     QSV_REQUIRE((size_t)channels * 4 <= 64 * 1024, "qsv_conv_silu_unit: %d channels do not fit the workgroup's LDS", channels);
     if (n_tokens == 0) return QSV_OK;
     QSV_DISPATCH(dtype, "qsv_conv_silu_unit",
                  hipLaunchKernelGGL(conv_silu_unit_kernel<T>, dim3(n_tokens), dim3(NT), (size_t)channels * 4, (hipStream_t)stream, out,
                                     (const T*)proj, stride, off, channels, taps, w, hist, run_off, state_rd, state_wr, n_unit,
-                                    unit_dim));
+                                    unit_dim, act));
     return qsv_launch_status("qsv_conv_silu_unit");
 }
 
@@ -700,4 +700,60 @@ extern "C" int qsv_rotate_heads(void* o, const float* rope, const int32_t* pos, 
                  hipLaunchKernelGGL(rotate_heads_kernel<T>, dim3(n_tokens), dim3(NT), 0, (hipStream_t)stream, (T*)o, rope, pos, sign,
                                     heads, n));
     return qsv_launch_status("qsv_rotate_heads");
+}
+
+
+// ---- element-wise gated recurrence (minGRU) ---------------------------------------------------------------------------------------
+// Thread = one channel of one run; the run's tokens are walked in order, UN at a time: the UN tokens' three pre-activations are
+// requested together (rows of the batch, coalesced over the channels), the gates are computed, then the UN dependent steps run.
+// Gates, candidate and state are float.
+template <typename T>
+__global__ __launch_bounds__(NT) void min_gru_scan_kernel(T* __restrict__ out, const T* __restrict__ proj, int64_t stride, int z_off,
+                                                          int x_off, int g_off, const T* __restrict__ b_z, const T* __restrict__ b_x,
+                                                          float* __restrict__ state, const int32_t* __restrict__ runs, int width) {
+    constexpr int UN = 8;
+    const int i = blockIdx.x * NT + threadIdx.x;
+    if (i >= width) return;
+    const int32_t* r = runs + 4 * blockIdx.y;
+    const int slot = r[0], first = r[1], n = r[2], p0 = r[3];
+    float S = p0 > 0 ? state[(size_t)slot * width + i] : 0.f;
+    const float bz = ld(b_z, i), bx = ld(b_x, i);
+    for (int t0 = 0; t0 < n; t0 += UN) {
+        float z[UN], u[UN], g[UN];
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const size_t row = (size_t)(first + min(t0 + j, n - 1)) * stride;
+            z[j] = ld(proj, row + z_off + i);
+            u[j] = ld(proj, row + x_off + i);
+            g[j] = ld(proj, row + g_off + i);
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            z[j] = 1.0f / (1.0f + expf(-(z[j] + bz)));
+            const float uu = u[j] + bx;
+            u[j] = uu >= 0.f ? uu + 0.5f : 1.0f / (1.0f + expf(-uu));
+            g[j] = g[j] / (1.0f + expf(-g[j]));
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            if (t0 + j < n) {
+                S = (1.0f - z[j]) * S + z[j] * u[j];
+                st(out, (size_t)(first + t0 + j) * width + i, S * g[j]);
+            }
+        }
+    }
+    state[(size_t)slot * width + i] = S;
+}
+extern "C" int qsv_min_gru_scan(void* out, const void* proj, int64_t stride, int z_off, int x_off, int g_off, const void* b_z,
+                                const void* b_x, float* state, const int32_t* runs, int n_runs, int width, int dtype, void* stream) {
+    QSV_REQUIRE(out && proj && b_z && b_x && state && runs, "qsv_min_gru_scan: null argument");
+    QSV_REQUIRE(width > 0 && n_runs >= 0 && n_runs <= 65535 && z_off >= 0 && x_off >= 0 && g_off >= 0 &&
+                    (int64_t)z_off + width <= stride && (int64_t)x_off + width <= stride && (int64_t)g_off + width <= stride,
+                "qsv_min_gru_scan: bad sizes");
+    if (n_runs == 0) return QSV_OK;
+    QSV_DISPATCH(dtype, "qsv_min_gru_scan",
+                 hipLaunchKernelGGL(min_gru_scan_kernel<T>, dim3((width + NT - 1) / NT, n_runs), dim3(NT), 0, (hipStream_t)stream,
+                                    (T*)out, (const T*)proj, stride, z_off, x_off, g_off, (const T*)b_z, (const T*)b_x, state, runs,
+                                    width));
+    return qsv_launch_status("qsv_min_gru_scan");
 }

@@ -425,3 +425,210 @@ extern "C" int qsv_normed_attention_prep(float* qf, void* pool, int64_t pool_row
                                     (const T*)k_w, eps, scale, (const T*)v_first, vf_stride, mix, slot));
     return qsv_launch_status("qsv_normed_attention_prep");
 }
+
+// ---- sublayers between two norms: x += rms_norm(y) * w_post; h = rms_norm(x) * w_next ---------------------------------------------
+// One workgroup per token, the row in registers (VPT groups of four values per thread; VPT = 0: any width, values re-read).  A
+// weight is one gain (wide 0) or one per coordinate.
+template <typename T>
+__device__ __forceinline__ float4 gain4(const T* w, int wide, int i) {
+    if (wide) return ld4v(w, i);
+    const float g = ld(w, 0);
+    return make_float4(g, g, g, g);
+}
+template <typename T, int VPT>
+__global__ __launch_bounds__(NT) void add_normed_rms_norm_vec_kernel(float* __restrict__ x, T* __restrict__ h, const T* __restrict__ y,
+                                                                     const T* __restrict__ w_post, int post_wide,
+                                                                     const T* __restrict__ w_next, int next_wide, float eps, int D) {
+    __shared__ float red[NT / 64 + 1];
+    const size_t t = blockIdx.x;
+    float4 v[VPT];
+    float s = 0.f;
+    if (y) {
+        float4 u[VPT];
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            const int i = (threadIdx.x + k * NT) * 4;
+            if (i >= D) continue;
+            u[k] = ld4v(y, t * D + i);
+            s += u[k].x * u[k].x + u[k].y * u[k].y + u[k].z * u[k].z + u[k].w * u[k].w;
+        }
+        const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
+        s = 0.f;
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            const int i = (threadIdx.x + k * NT) * 4;
+            if (i >= D) continue;
+            const float4 g = gain4(w_post, post_wide, i);
+            v[k] = ld4v(x, t * D + i);
+            v[k].x += u[k].x * inv * g.x; v[k].y += u[k].y * inv * g.y; v[k].z += u[k].z * inv * g.z; v[k].w += u[k].w * inv * g.w;
+            st4v(x, t * D + i, v[k]);
+            s += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+            const int i = (threadIdx.x + k * NT) * 4;
+            if (i >= D) continue;
+            v[k] = ld4v(x, t * D + i);
+            s += v[k].x * v[k].x + v[k].y * v[k].y + v[k].z * v[k].z + v[k].w * v[k].w;
+        }
+    }
+    if (!h) return;
+    const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+        const int i = (threadIdx.x + k * NT) * 4;
+        if (i >= D) continue;
+        const float4 g = gain4(w_next, next_wide, i);
+        st4v(h, t * D + i, make_float4(v[k].x * inv * g.x, v[k].y * inv * g.y, v[k].z * inv * g.z, v[k].w * inv * g.w));
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(NT) void add_normed_rms_norm_kernel(float* __restrict__ x, T* __restrict__ h, const T* __restrict__ y,
+                                                                 const T* __restrict__ w_post, int post_wide,
+                                                                 const T* __restrict__ w_next, int next_wide, float eps, int D) {
+    __shared__ float red[NT / 64 + 1];
+    const size_t t = blockIdx.x;
+    float s = 0.f;
+    if (y) {
+        for (int i = threadIdx.x; i < D; i += NT) {
+            const float u = ld(y, t * D + i);
+            s += u * u;
+        }
+        const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
+        s = 0.f;
+        for (int i = threadIdx.x; i < D; i += NT) {
+            const float v = x[t * D + i] + ld(y, t * D + i) * inv * ld(w_post, post_wide ? i : 0);
+            x[t * D + i] = v;
+            s += v * v;
+        }
+    } else {
+        for (int i = threadIdx.x; i < D; i += NT) s += x[t * D + i] * x[t * D + i];
+    }
+    if (!h) return;
+    const float inv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)D + eps);
+    for (int i = threadIdx.x; i < D; i += NT) st(h, t * D + i, x[t * D + i] * inv * ld(w_next, next_wide ? i : 0));
+}
+extern "C" int qsv_add_normed_rms_norm(float* x, void* h, const void* y, const void* w_post, int post_wide, const void* w_next,
+                                       int next_wide, float eps, int n, int D, int dtype, void* stream) {
+    QSV_REQUIRE(x && n >= 0 && D > 0 && (!h || w_next) && (!y || w_post), "qsv_add_normed_rms_norm: bad arguments");
+    if (n == 0) return QSV_OK;
+    const int vecs = (D / 4 + NT - 1) / NT;
+    if (D % 4 == 0 && vecs <= 8) {
+#define QSV_ANR(V)                                                                                                               \
+    QSV_DISPATCH(dtype, "qsv_add_normed_rms_norm",                                                                               \
+                 hipLaunchKernelGGL((add_normed_rms_norm_vec_kernel<T, V>), dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (T*)h, \
+                                    (const T*)y, (const T*)w_post, post_wide, (const T*)w_next, next_wide, eps, D))
+        if (vecs <= 1) QSV_ANR(1);
+        else if (vecs <= 2) QSV_ANR(2);
+        else if (vecs <= 4) QSV_ANR(4);
+        else QSV_ANR(8);
+#undef QSV_ANR
+        return qsv_launch_status("qsv_add_normed_rms_norm");
+    }
+    QSV_DISPATCH(dtype, "qsv_add_normed_rms_norm",
+                 hipLaunchKernelGGL(add_normed_rms_norm_kernel<T>, dim3(n), dim3(NT), 0, (hipStream_t)stream, x, (T*)h, (const T*)y,
+                                    (const T*)w_post, post_wide, (const T*)w_next, next_wide, eps, D));
+    return qsv_launch_status("qsv_add_normed_rms_norm");
+}
+
+// ---- query / key norms (per head or over the projection), rotated pairs, cache write -----------------------------------------------
+// One workgroup per token.  Statistics: per head a wave's sum over `dim`; over the projection a workgroup sum.  The rotation works
+// on normed values staged in LDS (a pair's two values may sit in different threads).  Dynamic LDS: (heads + kv_heads) * dim floats.
+template <typename T, typename TI>
+__global__ __launch_bounds__(NT) void qk_norm_rope_prep_kernel(float* __restrict__ qf, const TI* __restrict__ q, int64_t q_stride,
+                                                               const TI* __restrict__ k, int64_t k_stride, const TI* __restrict__ v,
+                                                               int64_t v_stride, int H, int G, int dim, int vdim,
+                                                               const T* __restrict__ q_w, const T* __restrict__ k_w, int per_head,
+                                                               float eps, const float* __restrict__ rope, int rot_n, float scale,
+                                                               T* __restrict__ pool, int64_t pool_rows,
+                                                               const int64_t* __restrict__ slot, const int32_t* __restrict__ pos) {
+    extern __shared__ float sm[];
+    __shared__ float red[NT / 64 + 1];
+    const size_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int NH = k ? H + G : H;                      // heads staged: the queries', then the keys'
+    float* nq = sm;                                    // [NH][dim]
+    const TI* qrow = q + t * q_stride;
+    const TI* krow = k ? k + t * k_stride : nullptr;
+    if (per_head) {
+        for (int hh = wv; hh < NH; hh += NT / 64) {
+            const TI* src = hh < H ? qrow + (size_t)hh * dim : krow + (size_t)(hh - H) * dim;
+            const T* w = hh < H ? q_w : k_w;
+            float s = 0.f;
+            for (int e = lane; e < dim; e += 64) {
+                const float u = ld(src, e);
+                s += u * u;
+            }
+            const float inv = 1.0f / sqrtf(wave_sum(s) / (float)dim + eps);
+            for (int e = lane; e < dim; e += 64) nq[hh * dim + e] = ld(src, e) * inv * ld(w, e);
+        }
+    } else {
+        float s = 0.f;
+        for (int i = threadIdx.x; i < H * dim; i += NT) {
+            const float u = ld(qrow, i);
+            s += u * u;
+        }
+        const float qinv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)(H * dim) + eps);
+        for (int i = threadIdx.x; i < H * dim; i += NT) nq[i] = ld(qrow, i) * qinv * ld(q_w, i);
+        if (k) {
+            s = 0.f;
+            for (int i = threadIdx.x; i < G * dim; i += NT) {
+                const float u = ld(krow, i);
+                s += u * u;
+            }
+            const float kinv = 1.0f / sqrtf(block_sum<NT>(s, red) / (float)(G * dim) + eps);
+            for (int i = threadIdx.x; i < G * dim; i += NT) nq[H * dim + i] = ld(krow, i) * kinv * ld(k_w, i);
+        }
+    }
+    __syncthreads();
+    if (rope) {                                        // pairs of neighbours, each by one thread
+        const int half = rot_n / 2;
+        const float* cs = rope + (size_t)pos[t] * rot_n;
+        for (int idx = threadIdx.x; idx < NH * half; idx += NT) {
+            const int hh = idx / half, i = idx - hh * half;
+            const float c = cs[i], sn = cs[half + i];
+            const float a = nq[hh * dim + 2 * i], b = nq[hh * dim + 2 * i + 1];
+            nq[hh * dim + 2 * i] = a * c - b * sn;
+            nq[hh * dim + 2 * i + 1] = b * c + a * sn;
+        }
+        __syncthreads();
+    }
+    const int R = vdim + dim;
+    for (int idx = threadIdx.x; idx < H * R; idx += NT) {
+        const int h = idx / R, c = idx - h * R;
+        qf[t * H * (size_t)R + idx] = c < vdim ? 0.f : nq[h * dim + c - vdim] * scale;
+    }
+    if (!k) return;
+    const size_t dst = (size_t)slot[t];
+    const TI* vrow = v + t * v_stride;
+    for (int idx = threadIdx.x; idx < G * R; idx += NT) {
+        const int g = idx / R, c = idx - g * R;
+        st(pool, ((size_t)g * pool_rows + dst) * R + c, c < vdim ? ld(vrow, g * vdim + c) : nq[(H + g) * dim + c - vdim]);
+    }
+}
+extern "C" int qsv_qk_norm_rope_prep(float* qf, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
+                                     int64_t v_stride, int qkv_dtype, int heads, int kv_heads, int dim, int vdim, const void* q_w,
+                                     const void* k_w, int per_head, float eps, const float* rope, int rot_n, float scale, void* pool,
+                                     int64_t pool_rows, const int64_t* slot, const int32_t* pos, int n, int dtype, void* stream) {
+    QSV_REQUIRE(qf && q && q_w && pos, "qsv_qk_norm_rope_prep: null argument");
+    QSV_REQUIRE(!k || (v && k_w && pool && slot), "qsv_qk_norm_rope_prep: keys without values, weight, pool or rows");
+    QSV_REQUIRE(heads > 0 && kv_heads > 0 && dim > 0 && vdim > 0 && n >= 0 && q_stride >= (int64_t)heads * dim &&
+                    (!k || (k_stride >= (int64_t)kv_heads * dim && v_stride >= (int64_t)kv_heads * vdim)),
+                "qsv_qk_norm_rope_prep: bad sizes");
+    QSV_REQUIRE(!rope || (rot_n > 0 && rot_n % 2 == 0 && rot_n <= dim), "qsv_qk_norm_rope_prep: %d rotated dimensions of %d", rot_n, dim);
+    QSV_REQUIRE(qkv_dtype == dtype || qkv_dtype == QSV_F32, "qsv_qk_norm_rope_prep: projections of type %d with storage type %d",
+                qkv_dtype, dtype);
+    const size_t lds = (size_t)(heads + kv_heads) * dim * 4;
+    QSV_REQUIRE(lds <= 64 * 1024, "qsv_qk_norm_rope_prep: %d + %d heads of %d do not fit the workgroup's LDS", heads, kv_heads, dim);
+    if (n == 0) return QSV_OK;
+#define QSV_QKP(TI)                                                                                                              \
+    QSV_DISPATCH(dtype, "qsv_qk_norm_rope_prep",                                                                                 \
+                 hipLaunchKernelGGL((qk_norm_rope_prep_kernel<T, TI>), dim3(n), dim3(NT), lds, (hipStream_t)stream, qf, (const TI*)q, \
+                                    q_stride, (const TI*)k, k_stride, (const TI*)v, v_stride, heads, kv_heads, dim, vdim,          \
+                                    (const T*)q_w, (const T*)k_w, per_head, eps, rope, rot_n, scale, (T*)pool, pool_rows, slot, pos))
+    if (qkv_dtype == QSV_F32) QSV_QKP(float);
+    else QSV_QKP(bf16_t);
+#undef QSV_QKP
+    return qsv_launch_status("qsv_qk_norm_rope_prep");
+}

@@ -212,12 +212,19 @@ __global__ __launch_bounds__(NT) void rms_pair_mean_kernel(T* __restrict__ out, 
         st(out, t * D + i, 0.5f * (ld(a, t * D + i) * ia * ld(wa, i) + ld(b, t * D + i) * ib * ld(wb, i)));
 }
 
-// out[r, f] = act(a[r, 2f]) * a[r, 2f + 1];  act 0: silu, 1: gelu in its tanh form, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))
+// out[r, f] = act(a[r, 2f]) * a[r, 2f + 1];  act 0: silu, 1: gelu in its tanh form, 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)));
+// act 2: g = min(gate, limit), u = clamp(up, -limit, limit) -> g sigmoid(1.702 g) (u + 1)
 template <typename T>
-__global__ __launch_bounds__(NT) void glu_kernel(T* __restrict__ out, const T* __restrict__ a, int ff, int act) {
+__global__ __launch_bounds__(NT) void glu_kernel(T* __restrict__ out, const T* __restrict__ a, int ff, int act, float limit) {
     const size_t r = blockIdx.x;
     for (int f = threadIdx.x; f < ff; f += NT) {
-        const float g = ld(a, (r * ff + f) * 2), u = ld(a, (r * ff + f) * 2 + 1);
+        float g = ld(a, (r * ff + f) * 2), u = ld(a, (r * ff + f) * 2 + 1);
+        if (act == 2) {
+            g = fminf(g, limit);
+            u = fminf(fmaxf(u, -limit), limit);
+            st(out, r * ff + f, g / (1.0f + expf(-1.702f * g)) * (u + 1.0f));
+            continue;
+        }
         const float ag = act == 0 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
         st(out, r * ff + f, ag * u);
     }
@@ -289,10 +296,10 @@ extern "C" int qsv_rms_pair_mean(void* out, const void* a, const void* wa, const
     return qsv_launch_status("qsv_rms_pair_mean");
 }
 
-extern "C" int qsv_glu(void* out, const void* a, int n_rows, int ff, int act, int dtype, void* stream) {
-    QSV_REQUIRE(out && a && n_rows >= 0 && ff > 0 && (act == 0 || act == 1), "qsv_glu: bad arguments");
+extern "C" int qsv_glu(void* out, const void* a, int n_rows, int ff, int act, float limit, int dtype, void* stream) {
+    QSV_REQUIRE(out && a && n_rows >= 0 && ff > 0 && (act == 0 || act == 1 || (act == 2 && limit > 0.f)), "qsv_glu: bad arguments");
     if (n_rows == 0) return QSV_OK;
     QSV_DISPATCH(dtype, "qsv_glu",
-                 hipLaunchKernelGGL(glu_kernel<T>, dim3(n_rows), dim3(NT), 0, (hipStream_t)stream, (T*)out, (const T*)a, ff, act));
+                 hipLaunchKernelGGL(glu_kernel<T>, dim3(n_rows), dim3(NT), 0, (hipStream_t)stream, (T*)out, (const T*)a, ff, act, limit));
     return qsv_launch_status("qsv_glu");
 }

@@ -17,30 +17,36 @@ SIGNATURES = {
     "qsv_layer_norm_rows": (_i, [_vp, _vp, _vp, _vp, _f, _i, _i, _i, _vp]),
     "qsv_latent_prep": (_i, [_vp, _i64, _i, _i, _vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _i, _vp]),
     "qsv_latent_query": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _i, _i, _i, _vp]),
-    "qsv_latent_attention": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _vp, _i, _i, _i, _vp]),
+    "qsv_latent_attention": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _vp, _i, _i, _vp, _vp, _i64, _i, _i,
+                                  _i, _i, _vp]),
+    "qsv_pool_blocks": (_i, [_vp, _i64, _vp, _i64, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "qsv_latent_attention_tile_tokens": (_i, [_i]),
     "qsv_latent_attention_mfma_ok": (_i, [_i, _i, _i]),
     "qsv_latent_attention_mfma": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _i, _i, _i64, _i, _vp,
-                                       _i, _vp]),
+                                       _i, _i, _vp, _vp, _i64, _i, _i, _vp]),
     "qsv_sigmoid_gate": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp]),
     "qsv_moe_route": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _f, _i, _vp]),
-    "qsv_moe_up": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp]),
-    "qsv_expert_rows": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "qsv_moe_up": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i, _i, _vp]),
+    "qsv_expert_rows": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp]),
     "qsv_grouped_gemm_tile_slots": (_i, []),
     "qsv_grouped_gemm_k_step": (_i, []),
-    "qsv_grouped_gemm": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "qsv_grouped_gemm": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _f, _vp]),
     "qsv_gather_rows": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "qsv_relu_sq": (_i, [_vp, _i64, _i, _vp]),
-    "qsv_moe_combine": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
-    "qsv_moe_down": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "qsv_moe_combine": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
+    "qsv_moe_down": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i, _i, _vp]),
     "qsv_embed_streams": (_i, [_vp, _vp, _vp, _f, _i, _i, _i, _i, _vp]),
     "qsv_hc_read": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "qsv_hc_write": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _vp]),
     "qsv_dyt_sum_rows": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _i, _vp]),
     "qsv_rms_pair_mean": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _i, _i, _i, _vp]),
-    "qsv_glu": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
+    "qsv_glu": (_i, [_vp, _vp, _i, _i, _i, _f, _i, _vp]),
     "qsv_decay": (_i, [_vp, _vp, _i64, _vp, _vp, _f, _i, _i, _i, _i, _vp]),
-    "qsv_conv_silu_unit": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "qsv_conv_silu_unit": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "qsv_min_gru_scan": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "qsv_add_normed_rms_norm": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _f, _i, _i, _i, _vp]),
+    "qsv_qk_norm_rope_prep": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _i, _vp, _vp, _i, _f, _vp, _i, _f, _vp, _i64,
+                                   _vp, _vp, _i, _i, _vp]),
     "qsv_recurrent_scan": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _vp, _vp, _i64, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _vp,
                                 _i, _i, _vp]),
     "qsv_head_rms_gate": (_i, [_vp, _vp, _vp, _vp, _i64, _i, _f, _i, _i, _i, _i, _i, _vp, _i, _vp]),

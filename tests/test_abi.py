@@ -96,9 +96,12 @@ def test_serve_argument_validation_without_gpu():
     assert L.qsv_moe_route(1, 1, 1, 1, None, 0, 4, 64, 8, 3, 4, 1, 0, None, 1, 1.0, 0, None) == 1  # top 3 of one kept group of 2
     assert b"experts" in L.qsv_last_error()
     assert L.qsv_moe_route(1, 1, 1, 1, None, 0, 4, 64, 8, 2, 4, 1, 2, None, 1, 1.0, 0, None) == 1  # unknown score function
-    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 1000, 1032, 64, 2, 0, 0, None, 0, 0, 1, None) == 1   # rows wider than 1024
-    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 64, 96, 64, 2, 0, -3, None, 0, 0, 1, None) == 1      # negative chunk
-    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 64, 96, 64, 2, 0, 0, 1, 0, 0, 1, None) == 1          # bias table without entries
+    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 1000, 1032, 64, 2, 0, 0, None, 0, 0, None, None, 0, 0, 0, 0, 1, None) == 1   # rows wider than 1024
+    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 64, 96, 64, 2, 0, -3, None, 0, 0, None, None, 0, 0, 0, 0, 1, None) == 1      # negative chunk
+    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 64, 96, 64, 2, 0, 0, 1, 0, 0, None, None, 0, 0, 0, 0, 1, None) == 1          # bias table without entries
+    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 0, 4, 2, 64, 96, 64, 2, 0, 0, None, 0, 5, None, None, 0, 0, 0, 0, 1, None) == 1      # kept first positions without a window
+    assert L.qsv_latent_attention(1, 1, 1, 1, 4, 1, 1, 32, 4, 2, 64, 96, 64, 2, 0, 0, None, 0, 0, None, 1, 0, 12, 5, 0, 1, None) == 1       # five block rows of 12 positions do not cover a page of 64
+    assert b"pooled" in L.qsv_last_error()
     assert L.qsv_latent_attention_mfma_ok(64, 80, 0) == 1 and L.qsv_latent_attention_mfma_ok(64, 80, 1) == 0
     assert L.qsv_latent_attention_mfma_ok(70, 70, 0) == 0
     assert [L.qsv_latent_attention_tile_tokens(h) for h in (1, 3, 6, 16, 32, 40)] == [64, 16, 8, 4, 4, 4]
@@ -107,10 +110,15 @@ def test_serve_argument_validation_without_gpu():
     assert L.qsv_recurrent_scan(1, 1, 8, 1, 8, 1, 8, 1, 1, None, 0, 0, 1, 1, 1, 5, 2, 2, 8, 8, 1.0, None, 1, 12, None) == 1  # more value columns than the state has
     assert L.qsv_head_rms_gate(1, 1, 1, 1, 16, 1, 1e-5, 2, 2, 8, 8, 1, 1, 0, None) == 1                       # a normaliser without its column
     assert L.qsv_max_gates(1, 1, 1, 1, 1, 4, 1, 1, 0.0, 1, 1, 1, 4, 0, None) == 1                             # gate cap 0
-    assert L.qsv_glu(1, 1, 2, 8, 7, 0, None) == 1                                                             # unknown activation
+    assert L.qsv_glu(1, 1, 2, 8, 7, 0.0, 0, None) == 1                                                        # unknown activation
+    assert L.qsv_glu(1, 1, 2, 8, 2, 0.0, 0, None) == 1                                                        # clamped units without a limit
     assert L.qsv_add_rms_norm(1, 1, None, None, None, None, 1e-5, 2, 8, 0, None) == 1                         # a norm without its weight
     assert L.qsv_hc_write(1, 1, 1, 1, 2, 17, 8, None, None, None, None, 0.0, 0, None) == 1                    # 17 streams
-    assert L.qsv_moe_up(1, 1, 1, 1, 1, 1, 8, 7, 2, 0, None) == 1                                              # gated units, odd rows
+    assert L.qsv_moe_up(1, 1, 1, 1, 1, 1, 8, 7, 2, 0.0, 4, 0, None) == 1                                      # gated units, odd rows
+    assert L.qsv_moe_up(1, 1, 1, 1, 1, 1, 8, 8, 3, 0.0, 4, 0, None) == 1                                      # clamped units without a limit
+    assert L.qsv_add_normed_rms_norm(1, 1, 1, None, 0, 1, 0, 1e-5, 2, 8, 0, None) == 1                        # an added sublayer output without its gain
+    assert L.qsv_qk_norm_rope_prep(1, 1, 64, None, 0, None, 0, 0, 2, 1, 32, 32, 1, None, 1, 1e-5, 1, 40, 1.0, None, 0, None, 1, 2, 0, None) == 1   # 40 rotated dimensions of 32
+    assert L.qsv_min_gru_scan(1, 1, 16, 0, 8, 16, 1, 1, 1, 1, 1, 8, 0, None) == 1                            # the gate's columns lie outside the rows
     with pytest.raises(RuntimeError):
         check(L.qsv_embed(0, 1, 1, 1, 1, 8, 0, None), "embed")
 
@@ -120,6 +128,6 @@ def test_serving_package_does_not_need_the_w4a8_library():
     the serving kernels."""
     import subprocess
     import sys
-    code = ("import sys; import qserve_amd.serving, qserve_amd.models.vekalorn, qserve_amd.models.mumelix, qserve_amd.models.vepolix, qserve_amd.serving.trace; "
+    code = ("import sys; import qserve_amd.serving, qserve_amd.models.vekalorn, qserve_amd.models.mumelix, qserve_amd.models.vepolix, qserve_amd.models.pemolorn, qserve_amd.serving.trace; "
             "bad = [m for m in sys.modules if m in ('qserve_amd._lib', 'qserve_amd.decode', 'qserve_backend')]; sys.exit(1 if bad else 0)")
     assert subprocess.run([sys.executable, "-c", code], cwd=ROOT).returncode == 0
