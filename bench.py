@@ -12,7 +12,7 @@ greedy sampling, replayed from a hipGraph.  N > 1 = tensor parallel over N GPUs 
 weights, 2 RCCL all-reduces per layer); default WEAK scaling (64 sequences per GPU, `--scaling strong` keeps the
 global batch).  `python bench.py --gpus N` without a launcher re-executes itself under torch.distributed.run.
 
-`--design vekalorn` / `--design mumelix` / `--design vepolix` run another workload altogether (prompt-phase and decode throughput of a design served by the paged engine
+`--design vekalorn` / `--design mumelix` / `--design vepolix` / `--design pemolorn` run another workload altogether (prompt-phase and decode throughput of a design served by the paged engine
 beside this Llama engine at equal size, one JSON line per size: qserve_amd/serving/bench.py); the default line is unchanged.
 
 `--config` selects the other BASELINE.json configurations (3: g128 bs=128; 4: Qwen1.5-72B TP=8 global bs=64, strong;
@@ -84,10 +84,10 @@ def parse():
     ap.add_argument("--scaling", default=None, choices=["weak", "strong"],
                     help="N>1 (tensor parallel): weak = --batch sequences PER GPU (global batch = batch x N, so every "
                          "rank keeps N=1's GEMM MACs and KV bytes); strong = --batch is the global batch")
-    ap.add_argument("--design", default=None, choices=["vekalorn", "mumelix", "vepolix"],
+    ap.add_argument("--design", default=None, choices=["vekalorn", "mumelix", "vepolix", "pemolorn"],
                     help="instead of the default workload: prompt-phase and decode throughput of a design served by the paged "
                          "engine (qserve_amd/serving) beside the closest existing model at equal size (vekalorn: the W4A8KV4 "
-                         "Llama engine; mumelix: Vekalorn; vepolix: Mumelix); one JSON line per size")
+                         "Llama engine; mumelix: Vekalorn; vepolix and pemolorn: Mumelix); one JSON line per size")
     ap.add_argument("--design-sizes", default="w2048,w2048r256,w4096", help="with --design: comma-separated size names (qserve_amd/serving/bench.py)")
     a = ap.parse_args()
     preset = CONFIGS[a.config] if a.config else CONFIGS[2]

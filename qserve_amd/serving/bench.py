@@ -3,6 +3,7 @@
     python bench.py --design vekalorn [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside the W4A8KV4 Llama engine
     python bench.py --design mumelix  [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside Vekalorn
     python bench.py --design vepolix  [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside Mumelix
+    python bench.py --design pemolorn [--design-sizes w2048,w4096] [--steps K] [--warmup W]     beside Mumelix
 
 Per size (random weights, 4 layers, vocabulary 32000): prompt phase = 8 prompts x 1024 tokens in one step through
 Engine.execute; decoding = 64 sequences at context 1024, one token each per step.  Beside them the Llama-style W4A8KV4
@@ -77,7 +78,8 @@ class OpTimer:
     NAMES = ("embed", "add_layer_norm", "layer_norm_rows", "latent_prep", "latent_query", "latent_attention", "sigmoid_gate",
              "moe_route", "moe_experts", "embed_streams", "hc_read", "hc_write", "dyt_sum_rows", "rms_pair_mean", "glu",
              "attention_prep", "rotate_heads", "decay", "conv_silu_unit", "recurrent_scan", "head_rms_gate", "embed_sinusoid",
-             "add_rms_norm", "rms_norm_rows", "normed_attention_prep", "max_gates")
+             "add_rms_norm", "rms_norm_rows", "normed_attention_prep", "max_gates", "add_normed_rms_norm", "qk_norm_rope_prep", "pool_blocks",
+             "min_gru_scan", "relu_sq")
 
     def __init__(self, ops):
         self.ops, self.events, self.calls, self.on = ops, [], [], False
@@ -92,7 +94,7 @@ class OpTimer:
         import importlib
         return [importlib.import_module("qserve_amd." + m) for m in
                 ("layers.latent_attention", "layers.moe", "layers.recurrent", "layers.softmax_attention", "models.vekalorn",
-                 "models.mumelix", "models.vepolix")]
+                 "models.mumelix", "models.vepolix", "models.pemolorn")]
 
     def _wrap(self, name, fn):
         def timed(*a, **k):
@@ -533,6 +535,154 @@ def bench_vepolix(name, s, dev, steps, warmup):
     return out
 
 
+# ---- Pemolorn ---------------------------------------------------------------------------------------------------------------
+PEMOLORN_WINDOW, PEMOLORN_POOL, PEMOLORN_KEEP = 512, 64, 64
+
+
+def pemolorn_config(s, m):
+    """Mumelix's sizes in Pemolorn's layers: the attention heads and cache rows of its parallel layers, a minGRU as wide as the model
+    beside them, the same experts (plus four identity experts).  Layers: parallel (window 512 + pooled blocks of 64, dense unit of the
+    active expert width), attention (window over the whole context, 64 kept tokens), parallel, attention on the second layer's cache."""
+    att = {"heads": m["a_heads"], "kv_heads": m["a_kv"], "dim": m["a_dim"], "vdim": m["a_vdim"], "scale": 1.0 / math.sqrt(m["a_dim"])}
+    moe = {"kind": "moe", "expert": {"ff": s["ff"], "limit": 7.0}, "router": {"experts": s["experts"], "identity": 4, "top": s["top"]}}
+    left = dict(att, conv=m["taps"], mask={"size": PEMOLORN_WINDOW, "pool": PEMOLORN_POOL}, rot={"base": 500000.0, "dims": m["rot"]})
+    p = {"type": "parallel", "mixer": {"left": left, "right": {"width": s["width"]}}}
+    a = {"type": "attention", "mixer": dict(att, mask={"size": 2048, "keep_first": PEMOLORN_KEEP}), "mlp": moe}
+    shared = {"type": "attention", "mixer": dict(a["mixer"], kv_from=1), "mlp": moe}
+    return {"architecture": "Pemolorn", "width": s["width"], "vocab": VOCAB, "norm": {"eps": 1e-5},
+            "layers": [dict(p, mlp={"kind": "dense", "ff": s["top"] * s["ff"]}), a, dict(p, mlp=moe), shared][:LAYERS]}
+
+
+def pemolorn_weights(cfg, dev, seed=0):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    D, V = cfg["width"], cfg["vocab"]
+
+    def mat(o, i, s=1.0):
+        return (torch.randn((o, i), device=dev, generator=g) * (s / math.sqrt(i))).bfloat16()
+
+    def vec(n, mean=1.0, s=0.1):
+        return (mean + s * torch.randn((n,), device=dev, generator=g)).bfloat16()
+
+    def one(mean=1.0):
+        return vec(1, mean).reshape(())
+
+    W = {"embed": torch.randn((V, D), device=dev, generator=g).bfloat16(), "head": mat(V, D), "final.norm": one()}
+    for i, L in enumerate(cfg["layers"]):
+        p, x = f"l{i}.", L["mixer"]
+        for n in ("norm1", "norm1b", "norm2", "norm2b"):
+            W[p + n] = one()
+
+        def attention(q, a, whole, own=True):
+            H, G, d, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            W.update({q + "q": mat(H * d, D), q + "o": mat(D, H * dv), q + "sink": vec(H, 0.0, 1.0), q + "q.norm": vec(H * d if whole else d)})
+            if own:
+                W.update({q + "k": mat(G * d, D), q + "v": mat(G * dv, D), q + "k.norm": vec(G * d if whole else d)})
+            if a.get("conv"):
+                W.update({q + "q.conv": mat(H * d, a["conv"]), q + "k.conv": mat(G * d, a["conv"]), q + "v.conv": mat(G * dv, a["conv"])})
+
+        if L["type"] == "parallel":
+            attention(p + "mix.left.", x["left"], True)
+            n, q = x["right"]["width"], p + "mix.right."
+            W.update({q + "z": mat(n, D), q + "x": mat(n, D), q + "g": mat(n, D), q + "o": mat(D, n), q + "z.b": vec(n, 0.0, 1.0),
+                      q + "x.b": vec(n, 0.0, 1.0), p + "mix.left.out": vec(D), p + "mix.right.out": vec(D)})
+        else:
+            attention(p + "mix.", x, False, own=x.get("kv_from") is None)
+        mlp, q = L["mlp"], p + "mlp."
+        if mlp["kind"] == "dense":
+            W[q + "up"], W[q + "down"] = mat(mlp["ff"], D), mat(D, mlp["ff"])
+        else:
+            r = mlp["router"]
+            for e in range(r["experts"]):
+                W[f"{q}e{e}.gate"], W[f"{q}e{e}.up"], W[f"{q}e{e}.down"] = mat(mlp["expert"]["ff"], D), mat(mlp["expert"]["ff"], D), mat(D, mlp["expert"]["ff"])
+            n = r["experts"] + r["identity"]
+            W[q + "router"], W[q + "correction"] = mat(n, D, 3.0), vec(n, 0.0, 0.02)
+    return W
+
+
+def bench_pemolorn(name, s, dev, steps, warmup):
+    from ..models.pemolorn import Pemolorn
+    from .engine import Engine
+    m = MUMELIX[name]
+    cfg = pemolorn_config(s, m)
+    NB, L, BP = 64, 1024, 8
+    eng = Engine(Pemolorn, cfg, pemolorn_weights(cfg, dev), dtype="bfloat16", device=dev, max_tokens=NB * (L + 384), max_seqs=NB)
+    timer = OpTimer(eng.ops)
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, VOCAB, (L,), generator=g).tolist() for _ in range(NB)]
+    slots = [eng.open_sequence() for _ in range(NB)]
+    stateless = ("latent_attention", "add_normed_rms_norm", "qk_norm_rope_prep", "pool_blocks", "rms_pair_mean")
+    pre_ms, ops_pre, rep_pre = [], None, {}
+    for i in range(0, NB, BP):
+        items = [(slots[j], prompts[j]) for j in range(i, i + BP)]
+        want = [k * L + L - 1 for k in range(BP)]
+        if i == BP:                                          # one step with events around every launch
+            ops_pre, _ = timer.step(lambda: eng.execute(items, want))
+            rep_pre = {k: timer.replay(k, 3) for k in stateless}      # (the scan and the convolution advance state: timed in the step)
+            continue
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        eng.execute(items, want)
+        torch.cuda.synchronize()
+        if i > 0:
+            pre_ms.append((time.perf_counter() - t0) * 1e3)
+    pre = sorted(pre_ms)[len(pre_ms) // 2]
+    nxt = [[int(torch.randint(0, VOCAB, (1,), generator=g))] for _ in range(NB)]
+    want = list(range(NB))
+
+    def decode():
+        eng.execute([(slots[j], nxt[j]) for j in range(NB)], want)
+
+    dec_eager = timed(decode, steps, warmup)
+    ops_dec, dec_events_ms = timer.step(decode)
+    rep_dec = {k: timer.replay(k, 20) for k in ("latent_attention", "moe_experts", "add_normed_rms_norm", "qk_norm_rope_prep")}
+    eng.decode_graphs = True
+    dec = timed(decode, steps, warmup)
+    graph_ok = any(v is not False for v in eng._graphs.values()) and bool(eng._graphs)
+    ctx = eng.cache.length[slots[0]]
+    T, D = BP * L, s["width"]
+    kinds = [x["type"] for x in cfg["layers"]]
+    n_par, n_att = kinds.count("parallel"), kinds.count("attention")
+    n_moe = sum(1 for x in cfg["layers"] if x["mlp"]["kind"] == "moe")
+    R = m["a_dim"] + m["a_vdim"]
+    W_, P_ = PEMOLORN_WINDOW, PEMOLORN_POOL
+
+    def seen(p, kind):                                       # keys a query at position p scores
+        return p + 1 if kind == "attention" else min(p + 1, W_) + max(0, p - W_ + 1) // P_
+
+    # attention: useful work = q.k over dim and p.v over vdim for every visible key (the kernel also multiplies the query's zero half)
+    att_flops = sum(BP * sum(seen(p, k) for p in range(L)) for k in kinds) * m["a_heads"] * R * 2.0
+    att_pre = att_flops / (rep_pre["latent_attention"] * 1e-3) / 1e12
+    att_bytes = sum(NB * seen(ctx - 1, k) for k in kinds) * m["a_kv"] * R * 2.0
+    att_dec = att_bytes / (rep_dec["latent_attention"] * 1e-3) / 1e9
+    # the element-wise recurrence moves three pre-activations in and one value out per token and channel (bfloat16)
+    scan_bytes = n_par * D * 4 * 2.0
+    scan_pre = T * scan_bytes / (ops_pre["min_gru_scan"] * 1e-3) / 1e9
+    scan_dec = NB * (scan_bytes + n_par * D * 8.0) / (ops_dec["min_gru_scan"] * 1e-3) / 1e9      # (+ the float state in and out)
+    active = s["top"] * s["experts"] / (s["experts"] + 4.0)  # chosen router outputs that are experts with weights, on average
+    moe_flops = n_moe * T * active * 3 * 2.0 * s["ff"] * D
+    moe_pre = moe_flops / (ops_pre["moe_experts"] * 1e-3) / 1e12
+    moe_bytes = n_moe * min(s["experts"], NB * s["top"]) * 3 * s["ff"] * D * 2.0
+    moe_dec = moe_bytes / (rep_dec["moe_experts"] * 1e-3) / 1e9
+    # residual kernel: per sublayer the float stream in and out, the sublayer's output in, the next input out; the first call only norms
+    res_bytes = T * (2 * LAYERS * (8.0 * D + 4.0 * D) + 4.0 * D + 2.0 * D)
+    res_pre = res_bytes / (rep_pre["add_normed_rms_norm"] * 1e-3) / 1e9
+    out = dict(model=f"Pemolorn-{name}", sizes=m, prefill_tokens_per_s=T / pre * 1e3, prefill_ms=pre, decode_tokens_per_s=NB / dec * 1e3,
+               decode_ms=dec, decode_from_hipgraph=graph_ok, decode_ms_eager=dec_eager, decode_ms_gpu_events=dec_events_ms, context=ctx,
+               prefill_ops_ms=ops_pre, decode_ops_ms=ops_dec, prefill_kernels_ms=rep_pre, decode_kernels_ms=rep_dec,
+               roofline=dict(prefill_attention_tflops=att_pre, prefill_attention_frac_bf16_peak=att_pre / BF16_PEAK_TFLOPS,
+                             decode_attention_gbs=att_dec, decode_attention_frac_hbm=att_dec / HBM_PEAK_GBS,
+                             prefill_experts_tflops=moe_pre, prefill_experts_frac_bf16_peak=moe_pre / BF16_PEAK_TFLOPS,
+                             decode_experts_gbs=moe_dec, decode_experts_frac_hbm=moe_dec / HBM_PEAK_GBS,
+                             prefill_recurrence_gbs=scan_pre, prefill_recurrence_frac_hbm=scan_pre / HBM_PEAK_GBS,
+                             decode_recurrence_gbs=scan_dec, decode_recurrence_frac_hbm=scan_dec / HBM_PEAK_GBS,
+                             prefill_residual_kernel_gbs=res_pre, prefill_residual_kernel_frac_hbm=res_pre / HBM_PEAK_GBS))
+    for sl in slots:
+        eng.close_sequence(sl)
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
 def main(args, helpers):
     dev = "cuda:0"
     torch.cuda.set_device(0)
@@ -542,12 +692,15 @@ def main(args, helpers):
         build.build(verbose=False)
     steps, warmup = min(args.steps, 32), min(args.warmup, 8)
     for name in args.design_sizes.split(","):
-        if args.design in ("mumelix", "vepolix") and name not in MUMELIX:      # (sizes that differ in a Vekalorn-only constant)
+        if args.design in ("mumelix", "vepolix", "pemolorn") and name not in MUMELIX:      # (sizes that differ in a Vekalorn-only constant)
             continue
         s = SIZES[name]
         line = {"design": args.design, "size": name, "sizes": s, "layers": LAYERS, "vocab": VOCAB, "dtype": "bf16",
                 "data": "synthetic", "workload": "prefill 8 x 1024 tokens in one step; decode 64 sequences at context 1024"}
-        if args.design == "vepolix":
+        if args.design == "pemolorn":
+            line["pemolorn"] = bench_pemolorn(name, s, dev, steps, warmup)
+            line["mumelix"] = bench_mumelix(name, s, dev, steps, warmup)
+        elif args.design == "vepolix":
             line["vepolix"] = bench_vepolix(name, s, dev, steps, warmup)
             line["mumelix"] = bench_mumelix(name, s, dev, steps, warmup)
         elif args.design == "mumelix":

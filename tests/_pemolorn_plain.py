@@ -194,3 +194,70 @@ def forward(config, W, tokens, taps=None, store=lambda a: a):
         if taps is not None:
             taps.append(x.copy())
     return (rms(x, eps) * W["final.norm"]) @ W["head"].T
+
+
+def tensor_shapes(config):
+    """name -> shape of every tensor a checkpoint of this config holds."""
+    D, V, out = config["width"], config["vocab"], {}
+    out["embed"], out["head"], out["final.norm"] = (V, D), (V, D), ()
+    for i, L in enumerate(config["layers"]):
+        p, m = f"l{i}.", L["mixer"]
+        for n in ("norm1", "norm1b"):
+            out[p + n] = ()
+
+        def attention(q, a, whole, own=True):
+            H, G, d, dv = a["heads"], a.get("kv_heads", a["heads"]), a["dim"], a["vdim"]
+            out[q + "q"], out[q + "o"], out[q + "sink"] = (H * d, D), (D, H * dv), (H,)
+            out[q + "q.norm"] = (H * d,) if whole else (d,)
+            if own:
+                out[q + "k"], out[q + "v"], out[q + "k.norm"] = (G * d, D), (G * dv, D), (G * d,) if whole else (d,)
+            if a.get("conv"):
+                out[q + "q.conv"], out[q + "k.conv"], out[q + "v.conv"] = (H * d, a["conv"]), (G * d, a["conv"]), (G * dv, a["conv"])
+
+        if L["type"] == "parallel":
+            attention(p + "mix.left.", m["left"], True)
+            n = m["right"]["width"]
+            for k in ("z", "x", "g"):
+                out[p + "mix.right." + k] = (n, D)
+            out[p + "mix.right.z.b"], out[p + "mix.right.x.b"], out[p + "mix.right.o"] = (n,), (n,), (D, n)
+            out[p + "mix.left.out"], out[p + "mix.right.out"] = (D,), (D,)
+        else:
+            attention(p + "mix.", m, False, own=m.get("kv_from") is None)
+        mlp = L.get("mlp")
+        if mlp:
+            out[p + "norm2"], out[p + "norm2b"] = (), ()
+            if mlp["kind"] == "dense":
+                out[p + "mlp.up"], out[p + "mlp.down"] = (mlp["ff"], D), (D, mlp["ff"])
+            else:
+                r, ff = mlp["router"], mlp["expert"]["ff"]
+                n = r["experts"] + r.get("identity", 0)
+                out[p + "mlp.router"], out[p + "mlp.correction"] = (n, D), (n,)
+                for e in range(r["experts"]):
+                    out[f"{p}mlp.e{e}.gate"], out[f"{p}mlp.e{e}.up"], out[f"{p}mlp.e{e}.down"] = (ff, D), (ff, D), (D, ff)
+    return out
+
+
+def random_weights(config, seed=0):
+    """Random tensors (numpy float64, every value a bfloat16 number) with scales that keep every mechanism awake: gains near 1,
+    sinks and corrections of the size of the scores they compete with."""
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    W = {}
+    for name, shape in tensor_shapes(config).items():
+        last = name.rsplit(".", 1)[-1]
+        if shape == () or last in ("norm", "out"):
+            t = 1.0 + 0.3 * torch.randn(shape, generator=g)
+        elif last == "sink":
+            t = torch.randn(shape, generator=g)
+        elif last == "correction":
+            t = 0.1 * torch.randn(shape, generator=g)
+        elif last == "b":
+            t = 0.5 * torch.randn(shape, generator=g)
+        elif last == "conv":
+            t = torch.randn(shape, generator=g) / math.sqrt(shape[1])
+        elif name in ("embed",):
+            t = torch.randn(shape, generator=g)
+        else:
+            t = torch.randn(shape, generator=g) / math.sqrt(shape[-1])
+        W[name] = t.bfloat16().double().numpy()
+    return W
