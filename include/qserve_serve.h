@@ -231,9 +231,11 @@ int qsv_conv_silu_unit(float* out, const void* proj, int64_t stride, int off, in
  * the others), further columns with zeros. */
 /* Element-wise gated recurrence over every run (slot, first token, tokens, first position): S = state[slot] (float [width], zeros
  * if the first position is 0), per token S <- (1 - z) S + z c with z = sigmoid(proj[t, z_off + i] + b_z[i]), u = proj[t, x_off + i] +
- * b_x[i], c = u + 1/2 if u >= 0 else sigmoid(u); out[t, i] = S * silu(proj[t, g_off + i]) (storage type); S is written back. */
+ * b_x[i], c = u + 1/2 if u >= 0 else sigmoid(u); out[t, i] = S * silu(proj[t, g_off + i]) (storage type); S is written back.
+ * max_run: the longest run's tokens as the host knows them (0: unknown); up to 32 a thread walks its channel's run, above that the
+ * run's segments are scanned side by side and composed. */
 int qsv_min_gru_scan(void* out, const void* proj, int64_t stride, int z_off, int x_off, int g_off, const void* b_z, const void* b_x,
-                     float* state, const int32_t* runs, int n_runs, int width, int dtype, void* stream);
+                     float* state, const int32_t* runs, int n_runs, int max_run, int width, int dtype, void* stream);
 int qsv_recurrent_scan(float* o, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v,
                        int64_t v_stride, int qkv_dtype, const float* decay, const void* beta, int64_t beta_stride,
                        int beta_dtype, float* state, const int32_t* runs, int n_runs, int max_run, int heads, int qk_heads,

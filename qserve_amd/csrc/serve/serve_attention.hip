@@ -200,6 +200,60 @@ __global__ __launch_bounds__(256) void pool_blocks_kernel(T* __restrict__ pooled
         st(dst, c, a * inv);
     }
 }
+// The same for rows that are whole 16-byte pieces (VEC elements each) and at most 256 pieces wide: a row's pieces side by side over
+// the lanes, the block's rows dealt to 256 / pieces row groups that sum their share at once; the groups' sums meet in LDS.
+__device__ __forceinline__ void load_piece(const float* p, float (&v)[4]) {
+    const float4 a = *(const float4*)p;
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+}
+__device__ __forceinline__ void load_piece(const bf16_t* p, float (&v)[8]) {
+    const uint4 u = *(const uint4*)p;
+    const unsigned w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void pool_blocks_vec_kernel(T* __restrict__ pooled, int64_t pooled_rows, const T* __restrict__ pool,
+                                                              int64_t pool_rows, const int32_t* __restrict__ block_table,
+                                                              int table_stride, const int32_t* __restrict__ seq,
+                                                              const int32_t* __restrict__ pos, int R, int pool_block, int page,
+                                                              int block_rows) {
+    __shared__ float part[256][VEC];
+    const size_t t = blockIdx.x;
+    const int g = blockIdx.y;
+    const int p = pos[t];
+    if ((p + 1) % pool_block) return;                       // (the whole workgroup)
+    const int32_t* bt = block_table + (size_t)seq[t] * table_stride;
+    const int first = p + 1 - pool_block;
+    const int pieces = R / VEC, groups = 256 / pieces;
+    const int col = threadIdx.x % pieces, grp = threadIdx.x / pieces;
+    const T* src = pool + (size_t)g * pool_rows * R;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    if (grp < groups) {
+        for (int j = first + grp; j <= p; j += groups) {
+            float v[VEC];
+            load_piece(src + ((size_t)bt[j / page] * page + (size_t)(j % page)) * R + col * VEC, v);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) part[threadIdx.x][e] = acc[e];
+    __syncthreads();
+    if (grp != 0) return;
+    for (int k = 1; k < groups; ++k)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) acc[e] += part[k * pieces + col][e];
+    T* dst = pooled + ((size_t)g * pooled_rows + (size_t)bt[first / page] * block_rows + (size_t)((first % page) / pool_block)) * R;
+    const float inv = 1.0f / (float)pool_block;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) st(dst, col * VEC + e, acc[e] * inv);
+}
 extern "C" int qsv_pool_blocks(void* pooled, int64_t pooled_rows, const void* pool, int64_t pool_rows, const int32_t* block_table,
                                int table_stride, const int32_t* seq, const int32_t* pos, int n, int n_pools, int R, int pool_block,
                                int page, int block_rows, int dtype, void* stream) {
@@ -208,6 +262,16 @@ extern "C" int qsv_pool_blocks(void* pooled, int64_t pooled_rows, const void* po
                     (int64_t)block_rows * pool_block >= page && table_stride > 0,
                 "qsv_pool_blocks: blocks of %d positions, %d rows per page of %d", pool_block, block_rows, page);
     if (n == 0) return QSV_OK;
+    if (dtype == QSV_BF16 && R % 8 == 0 && R / 8 <= 256) {
+        hipLaunchKernelGGL((pool_blocks_vec_kernel<bf16_t, 8>), dim3(n, n_pools), dim3(256), 0, (hipStream_t)stream, (bf16_t*)pooled,
+                           pooled_rows, (const bf16_t*)pool, pool_rows, block_table, table_stride, seq, pos, R, pool_block, page, block_rows);
+        return qsv_launch_status("qsv_pool_blocks");
+    }
+    if (dtype == QSV_F32 && R % 4 == 0 && R / 4 <= 256) {
+        hipLaunchKernelGGL((pool_blocks_vec_kernel<float, 4>), dim3(n, n_pools), dim3(256), 0, (hipStream_t)stream, (float*)pooled,
+                           pooled_rows, (const float*)pool, pool_rows, block_table, table_stride, seq, pos, R, pool_block, page, block_rows);
+        return qsv_launch_status("qsv_pool_blocks");
+    }
     QSV_DISPATCH(dtype, "qsv_pool_blocks",
                  hipLaunchKernelGGL(pool_blocks_kernel<T>, dim3(n, n_pools), dim3(256), 0, (hipStream_t)stream, (T*)pooled, pooled_rows,
                                     (const T*)pool, pool_rows, block_table, table_stride, seq, pos, R, pool_block, page, block_rows));

@@ -744,13 +744,92 @@ __global__ __launch_bounds__(NT) void min_gru_scan_kernel(T* __restrict__ out, c
     }
     state[(size_t)slot * width + i] = S;
 }
+// Long runs (prompt portions): a workgroup of SEG waves owns 64 channels of one run and cuts the run's tokens into SEG segments, one
+// a wave.  The recurrence S <- a S + b (a = 1 - z, b = z c) composes: a segment as a whole maps S to A S + B with A the product of
+// its a and B its own scan from zero.  Pass 1: every wave walks its segment for (A, B); the waves exchange them through LDS and each
+// folds its predecessors' into the state its segment starts from; pass 2: the segment again (from L2), now with outputs.
+template <typename T>
+__global__ __launch_bounds__(64 * 8) void min_gru_scan_segments_kernel(T* __restrict__ out, const T* __restrict__ proj, int64_t stride,
+                                                                       int z_off, int x_off, int g_off, const T* __restrict__ b_z,
+                                                                       const T* __restrict__ b_x, float* __restrict__ state,
+                                                                       const int32_t* __restrict__ runs, int width) {
+    constexpr int SEG = 8, UN = 8;
+    __shared__ float sA[SEG][64], sB[SEG][64];
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int ch = blockIdx.x * 64 + lane;
+    const bool valid = ch < width;
+    const int i = valid ? ch : width - 1;
+    const int32_t* r = runs + 4 * blockIdx.y;
+    const int slot = r[0], first = r[1], n = r[2], p0 = r[3];
+    const int per = (n + SEG - 1) / SEG;
+    const int t_lo = min(n, w * per), t_hi = min(n, t_lo + per);
+    const float bz = ld(b_z, i), bx = ld(b_x, i);
+    float A = 1.f, B = 0.f;
+    for (int t0 = t_lo; t0 < t_hi; t0 += UN) {
+        float z[UN], u[UN];
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const size_t row = (size_t)(first + min(t0 + j, t_hi - 1)) * stride;
+            z[j] = ld(proj, row + z_off + i);
+            u[j] = ld(proj, row + x_off + i);
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const float zz = 1.0f / (1.0f + expf(-(z[j] + bz)));
+            const float uu = u[j] + bx;
+            const float c = uu >= 0.f ? uu + 0.5f : 1.0f / (1.0f + expf(-uu));
+            if (t0 + j < t_hi) {
+                A *= 1.0f - zz;
+                B = (1.0f - zz) * B + zz * c;
+            }
+        }
+    }
+    sA[w][lane] = A;
+    sB[w][lane] = B;
+    __syncthreads();
+    float S = p0 > 0 ? state[(size_t)slot * width + i] : 0.f;
+    for (int k = 0; k < w; ++k) S = sA[k][lane] * S + sB[k][lane];
+    for (int t0 = t_lo; t0 < t_hi; t0 += UN) {
+        float z[UN], u[UN], g[UN];
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const size_t row = (size_t)(first + min(t0 + j, t_hi - 1)) * stride;
+            z[j] = ld(proj, row + z_off + i);
+            u[j] = ld(proj, row + x_off + i);
+            g[j] = ld(proj, row + g_off + i);
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            z[j] = 1.0f / (1.0f + expf(-(z[j] + bz)));
+            const float uu = u[j] + bx;
+            u[j] = uu >= 0.f ? uu + 0.5f : 1.0f / (1.0f + expf(-uu));
+            g[j] = g[j] / (1.0f + expf(-g[j]));
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            if (t0 + j < t_hi) {
+                S = (1.0f - z[j]) * S + z[j] * u[j];
+                if (valid) st(out, (size_t)(first + t0 + j) * width + i, S * g[j]);
+            }
+        }
+    }
+    if (w == SEG - 1 && valid) state[(size_t)slot * width + i] = S;     // (the last wave ends with the run's last state, also if its segment is empty)
+}
 extern "C" int qsv_min_gru_scan(void* out, const void* proj, int64_t stride, int z_off, int x_off, int g_off, const void* b_z,
-                                const void* b_x, float* state, const int32_t* runs, int n_runs, int width, int dtype, void* stream) {
+                                const void* b_x, float* state, const int32_t* runs, int n_runs, int max_run, int width, int dtype,
+                                void* stream) {
     QSV_REQUIRE(out && proj && b_z && b_x && state && runs, "qsv_min_gru_scan: null argument");
     QSV_REQUIRE(width > 0 && n_runs >= 0 && n_runs <= 65535 && z_off >= 0 && x_off >= 0 && g_off >= 0 &&
                     (int64_t)z_off + width <= stride && (int64_t)x_off + width <= stride && (int64_t)g_off + width <= stride,
                 "qsv_min_gru_scan: bad sizes");
     if (n_runs == 0) return QSV_OK;
+    if (max_run <= 0 || max_run > 32) {          // (0: unknown) long runs: segments of the run side by side
+        QSV_DISPATCH(dtype, "qsv_min_gru_scan",
+                     hipLaunchKernelGGL(min_gru_scan_segments_kernel<T>, dim3((width + 63) / 64, n_runs), dim3(64 * 8), 0,
+                                        (hipStream_t)stream, (T*)out, (const T*)proj, stride, z_off, x_off, g_off, (const T*)b_z,
+                                        (const T*)b_x, state, runs, width));
+        return qsv_launch_status("qsv_min_gru_scan");
+    }
     QSV_DISPATCH(dtype, "qsv_min_gru_scan",
                  hipLaunchKernelGGL(min_gru_scan_kernel<T>, dim3((width + NT - 1) / NT, n_runs), dim3(NT), 0, (hipStream_t)stream,
                                     (T*)out, (const T*)proj, stride, z_off, x_off, g_off, (const T*)b_z, (const T*)b_x, state, runs,

@@ -378,8 +378,8 @@ class HipOps:
         assert state.shape[1:] == (width,) and b_z.numel() == b_x.numel() == width and max(z_off, x_off, g_off) + width <= proj.size(1)
         runs = batch.runs()
         self.check(self.L.qsv_min_gru_scan(out.data_ptr(), proj.data_ptr(), proj.stride(0), z_off, x_off, g_off, b_z.data_ptr(),
-                                           b_x.data_ptr(), state.data_ptr(), runs.data_ptr(), runs.size(0), width, self.code,
-                                           self._s()), "min_gru_scan")
+                                           b_x.data_ptr(), state.data_ptr(), runs.data_ptr(), runs.size(0),
+                                           max(n for _, _, n in batch.items), width, self.code, self._s()), "min_gru_scan")
         return out
 
     # ---- recurrences ----------------------------------------------------------------------------------------------------------

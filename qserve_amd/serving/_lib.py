@@ -43,7 +43,7 @@ SIGNATURES = {
     "qsv_glu": (_i, [_vp, _vp, _i, _i, _i, _f, _i, _vp]),
     "qsv_decay": (_i, [_vp, _vp, _i64, _vp, _vp, _f, _i, _i, _i, _i, _vp]),
     "qsv_conv_silu_unit": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
-    "qsv_min_gru_scan": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "qsv_min_gru_scan": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "qsv_add_normed_rms_norm": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _i, _f, _i, _i, _i, _vp]),
     "qsv_qk_norm_rope_prep": (_i, [_vp, _vp, _i64, _vp, _i64, _vp, _i64, _i, _i, _i, _i, _i, _vp, _vp, _i, _f, _vp, _i, _f, _vp, _i64,
                                    _vp, _vp, _i, _i, _vp]),

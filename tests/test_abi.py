@@ -118,7 +118,7 @@ def test_serve_argument_validation_without_gpu():
     assert L.qsv_moe_up(1, 1, 1, 1, 1, 1, 8, 8, 3, 0.0, 4, 0, None) == 1                                      # clamped units without a limit
     assert L.qsv_add_normed_rms_norm(1, 1, 1, None, 0, 1, 0, 1e-5, 2, 8, 0, None) == 1                        # an added sublayer output without its gain
     assert L.qsv_qk_norm_rope_prep(1, 1, 64, None, 0, None, 0, 0, 2, 1, 32, 32, 1, None, 1, 1e-5, 1, 40, 1.0, None, 0, None, 1, 2, 0, None) == 1   # 40 rotated dimensions of 32
-    assert L.qsv_min_gru_scan(1, 1, 16, 0, 8, 16, 1, 1, 1, 1, 1, 8, 0, None) == 1                            # the gate's columns lie outside the rows
+    assert L.qsv_min_gru_scan(1, 1, 16, 0, 8, 16, 1, 1, 1, 1, 1, 1, 8, 0, None) == 1                            # the gate's columns lie outside the rows
     with pytest.raises(RuntimeError):
         check(L.qsv_embed(0, 1, 1, 1, 1, 8, 0, None), "embed")
 

@@ -520,12 +520,13 @@ def test_the_sink_takes_its_share(backend, dtype, tol):
                 assert (ref[0, :8] - h[0, 24:32]).abs().max() < 1e-6
 
 
-def test_pooled_rows_live_in_their_blocks_first_page(backend):
+@pytest.mark.parametrize("R", [6, 8, 1028])
+def test_pooled_rows_live_in_their_blocks_first_page(backend, R):
     """Blocks of 12 positions on pages of 64: the block [60, 72) straddles two pages and its row belongs to the first; six rows a
     page.  The rows hold the float mean of the cached rows."""
     dev = device_of(backend)
     ops = make_ops(backend, torch.float32, dev)
-    G, R, P_, page = 2, 6, 12, 64
+    G, P_, page = 2, 12, 64
     cache = PagedCache([(G, R), (G, R, 6)], 5, 2, torch.float32, dev, page=page)
     assert cache.pools[1].shape == (G, 5 * 6, R)
     cache.free_pages = [1, 4, 0, 3, 2]                                     # handed out from the end: 2, 3, 0
