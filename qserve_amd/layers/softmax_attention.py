@@ -132,7 +132,8 @@ class SinkWindowAttention:
     * rotary (a RotaryTable): the first rotary.dims dimensions of every q and k head turn with the position, neighbours paired.
     * keep_first: the first that many positions stay visible to every later query, at their true positions.
     * pool_block = P: beside the window's tokens a query at i sees one key and one value per block [bP, bP + P) that ends at or
-      before i - window: the means of the block's cached keys and values (a second pool, ceil(page / P) rows per page).
+      before i - window: the means of the block's cached keys and values (a second pool, ceil(page / P) rows per page, held by
+      the page of the block's first position).
     * shared_kv: the layer has no keys and values of its own and reads the pools of another layer of the same head counts.
     Cache: per key / value head one pool of rows [v | k] (k after norm and rotation), as the row-attention kernels read them."""
 
@@ -146,7 +147,7 @@ class SinkWindowAttention:
             raise ValueError("attention: a layer that reads another layer's keys and values has no convolution or pooled blocks")
         if pool_block and keep_first:
             raise ValueError("attention: pooled blocks and kept first tokens are alternatives")
-        if pool_block and not 0 < int(pool_block) <= page * 64:
+        if pool_block and int(pool_block) < 1:
             raise ValueError(f"attention: pooled blocks of {pool_block} positions")
         self.ops, self.H, self.G, self.dim, self.vdim, self.page = ops, heads, kv_heads, dim, vdim, page
         self.scale, self.eps, self.window, self.keep_first = float(scale), float(eps), int(window), int(keep_first or 0)
@@ -174,8 +175,7 @@ class SinkWindowAttention:
         if not shared_kv:
             self.cache_rows.append((kv_heads, R))
             if self.pool_block:
-                if self.pool_block > page:
-                    raise ValueError(f"attention: pooled blocks of {self.pool_block} positions on pages of {page}")
+                # (blocks longer than a page: at most one block starts in a page, one row a page)
                 self.cache_rows.append((kv_heads, R, (page + self.pool_block - 1) // self.pool_block))
         if self.taps and self.taps > 1:
             from ..serving.cache import StateSpec

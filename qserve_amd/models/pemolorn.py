@@ -86,9 +86,10 @@ class Pemolorn:
             if kind == "attention":
                 if m.get("kv_from") is not None:
                     src = int(m["kv_from"])
-                    if not 0 <= src < i or layers[src]["kv_from"] is not None or config["layers"][src]["type"] != "attention":
+                    if not 0 <= src < i or layers[src]["kv_from"] is not None:
                         raise ValueError(f"layer {i}: keys and values from layer {src}, which has none of its own before this layer")
                     other = config["layers"][src]["mixer"]
+                    other = other.get("left", other)                # (a parallel layer's cache is its attention's)
                     if any(int(other[k]) != int(m[k]) for k in ("kv_heads", "dim", "vdim")):
                         raise ValueError(f"layer {i}: layer {src}'s keys and values have other sizes")
                 mixer = attention(m, p, norm="head", shared_kv=src is not None)

@@ -95,7 +95,7 @@ def min_gru(h, w):
 
 def left_mixer(h, w, m, eps, store=lambda a: a):
     """The convolved, normed, rotated attention over a window and pooled blocks.  w: q, k, v, q_conv, k_conv, v_conv, q_norm,
-    k_norm, sink, o; m: the mixer's config."""
+    k_norm, sink, o; m: the mixer's config.  -> (output, (k, v) as a cache would hold them)."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     q, k, v = (short_conv(h @ w[n].T, w[n + "_conv"]) for n in ("q", "k", "v"))
@@ -105,8 +105,9 @@ def left_mixer(h, w, m, eps, store=lambda a: a):
     q, k = q.reshape(T, H, d), k.reshape(T, G, d)
     if rot:
         q, k = rotate_pairs(q, pos, rot["dims"], rot["base"]), rotate_pairs(k, pos, rot["dims"], rot["base"])
-    o = attention_pooled_blocks(q, k, v.reshape(T, G, dv), w["sink"], m["scale"], m["mask"]["size"], m["mask"]["pool"], store)
-    return o.reshape(T, H * dv) @ w["o"].T
+    v = v.reshape(T, G, dv)
+    o = attention_pooled_blocks(q, k, v, w["sink"], m["scale"], m["mask"]["size"], m["mask"]["pool"], store)
+    return o.reshape(T, H * dv) @ w["o"].T, (k, v)
 
 
 def attention_mixer(h, w, m, eps, shared=None, store=lambda a: a):
@@ -164,7 +165,7 @@ def forward(config, W, tokens, taps=None, store=lambda a: a):
             wl.update({n + "_conv": W[a + n + ".conv"] for n in ("q", "k", "v")}, q_norm=W[a + "q.norm"], k_norm=W[a + "k.norm"])
             wr = {n: W[b + n] for n in ("z", "x", "g", "o")}
             wr.update(z_b=W[b + "z.b"], x_b=W[b + "x.b"])
-            left, right = left_mixer(h, wl, m["left"], eps, store), min_gru(h, wr)
+            (left, cached[i]), right = left_mixer(h, wl, m["left"], eps, store), min_gru(h, wr)
             y = 0.5 * (rms(left, eps) * W[a + "out"] + rms(right, eps) * W[b + "out"])
         elif L["type"] == "attention":
             a = p + "mix."

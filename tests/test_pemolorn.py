@@ -239,7 +239,7 @@ def _mixer_alone(backend, layer, T, splits, seed=3, width=24, tol=2e-5, dtype="f
         wl.update({n + "_conv": W[a + n + ".conv"] for n in ("q", "k", "v")}, q_norm=W[a + "q.norm"], k_norm=W[a + "k.norm"])
         wr = {n: W[b + n] for n in ("z", "x", "g", "o")}
         wr.update(z_b=W[b + "z.b"], x_b=W[b + "x.b"])
-        ref = 0.5 * (P.rms(P.left_mixer(hd, wl, m["left"], eps), eps) * W[a + "out"] + P.rms(P.min_gru(hd, wr), eps) * W[b + "out"])
+        ref = 0.5 * (P.rms(P.left_mixer(hd, wl, m["left"], eps)[0], eps) * W[a + "out"] + P.rms(P.min_gru(hd, wr), eps) * W[b + "out"])
     else:
         wa = {n: W[p + n] for n in ("q", "k", "v", "sink", "o")}
         wa.update(q_norm=W[p + "q.norm"], k_norm=W[p + "k.norm"])
@@ -272,6 +272,7 @@ def test_pooled_block_attention_beside_min_gru_alone(backend):
     _mixer_alone(backend, par(heads=3, kv_heads=1, dim=10, vdim=6, size=1, pool=1, conv=4, rot=2, width=50), 40, [3, 4, 20])   # every earlier token is a block
     _mixer_alone(backend, par(heads=4, kv_heads=2, dim=4, vdim=12, size=30, pool=7, conv=1, rot=4, width=70), 200, [6, 7, 63, 64, 65, 69, 70, 140])
     _mixer_alone(backend, par(heads=2, kv_heads=1, dim=8, vdim=8, size=5, pool=50, conv=3, rot=8, width=12), 170, [49, 50, 54, 55, 56, 104, 105, 106])
+    _mixer_alone(backend, par(heads=2, kv_heads=2, dim=4, vdim=4, size=3, pool=70, conv=2, rot=2, width=6), 300, [69, 70, 72, 73, 139, 140, 143, 280])  # blocks longer than a page
 
 
 @pytest.mark.gpu
@@ -442,7 +443,7 @@ def _selector(backend, L, dtype, nq, *, spike=None, keep=0, size=50, pool=None, 
     if whole:
         one = np.zeros((1, 1))
         one[0, 0] = 1.0
-        ref = P.left_mixer(hn, dict(W, q_conv=np.ones((16, 1)), k_conv=np.ones((8, 1)), v_conv=np.ones((8, 1))), m, 1e-5)
+        ref = P.left_mixer(hn, dict(W, q_conv=np.ones((16, 1)), k_conv=np.ones((8, 1)), v_conv=np.ones((8, 1))), m, 1e-5)[0]
     else:
         ref = P.attention_mixer(hn, W, m, 1e-5)[0]
     dev = device_of(backend)
@@ -679,7 +680,8 @@ def test_other_sizes(backend, variant):
           att(heads=3, kv_heads=3, dim=16, vdim=24, size=64, keep=1, kv_from=0, mlp=None)], dict(width=96, vocab=200)),
         ([att(heads=2, kv_heads=2, dim=6, vdim=64, size=10, keep=2, mlp=None), par(heads=7, kv_heads=1, dim=70, vdim=5, size=3, pool=2, conv=2, rot=10, width=13)],
          dict(width=41, vocab=33, eps=1e-6)),
-        ([par(mlp=dense(8)), par(size=12, pool=12, mlp=moe(experts=8, identity=8, top=3)), att(heads=1, kv_heads=1, mlp=None), att(heads=5, kv_heads=1, kv_from=2)],
+        ([par(mlp=dense(8)), par(size=12, pool=12, mlp=moe(experts=8, identity=8, top=3)), att(heads=1, kv_heads=1, mlp=None), att(heads=5, kv_heads=1, kv_from=2),
+          att(heads=3, kv_heads=3, dim=8, vdim=10, size=200, keep=0, kv_from=0)],
          dict(width=48, vocab=61)),
     ][variant]
     cfg = make_config(layers, **kw)
@@ -712,7 +714,7 @@ def test_a_layer_without_keys_reads_its_source_layers_pools(backend, std):
     assert m.slices[2][:2] == m.slices[1][:2] and m.slices[5][:2] == m.slices[4][:2]
     assert m.layers[2]["mixer"].cache_rows == [] and len(eng.cache.pools) == 2 + 1 + 2 + 1      # two pools per pooled layer, one per owner
     bad = json.loads(json.dumps(cfg))
-    bad["layers"][2]["mixer"]["kv_from"] = 3                                                    # a later layer / not an attention layer
+    bad["layers"][2]["mixer"]["kv_from"] = 3                                                    # a later layer
     with pytest.raises(ValueError):
         Pemolorn.from_config(bad, f32(W), make_ops("unfused", torch.float32, "cpu"), "cpu", torch.float32)
 
