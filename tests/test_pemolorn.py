@@ -358,6 +358,33 @@ def test_router_with_identity_experts_alone(backend):
             assert_close(layer(h[lo:hi].to(dev)).double().cpu(), ref[lo:hi], 2e-5, f"{E} experts + {ident} identity, top {top}, tokens {lo}:{hi}")
 
 
+@pytest.mark.gpu
+def test_expert_kernel_forms_in_bfloat16():
+    """bfloat16 storage at sizes that take each form of the expert kernels (per token, expert-major, grouped on the matrix cores, vendor
+    products per expert): clamped units and identity experts in all of them.  The router reads the same bfloat16 input as the plain
+    statement, so the choices agree and only rounding is left."""
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    dev = "cuda:0"
+    ops = make_ops("hip", torch.bfloat16, dev)
+    g = torch.Generator().manual_seed(21)
+    for E, ident, top, D, ff, limit in ((6, 2, 3, 64, 64, 1.25), (5, 3, 2, 40, 24, 0.75), (30, 6, 4, 128, 64, 2.0)):
+        T = 700
+        h = torch.randn(T, D, generator=g).bfloat16()
+        router = (torch.randn(E + ident, D, generator=g) * 0.6).bfloat16()
+        corr = (torch.randn(E + ident, generator=g) * 0.05).bfloat16()
+        ex = [tuple((torch.randn(s_, generator=g) / 3).bfloat16() for s_ in ((ff, D), (ff, D), (D, ff))) for _ in range(E)]
+        ref = torch.from_numpy(P.moe_ff(h.double().numpy(), {"router": router.double().numpy(), "correction": corr.double().numpy(),
+                                                             "experts": [tuple(t.double().numpy() for t in e) for e in ex]}, top, ident, limit))
+        layer = IdentityExpertMoE(ops, router=router.to(dev), correction=corr.to(dev), gate=[e[0].to(dev) for e in ex],
+                                  up=[e[1].to(dev) for e in ex], down=[e[2].to(dev) for e in ex], top_k=top, identity=ident, limit=limit)
+        for lo, hi in ((0, 1), (1, 3), (3, 40), (40, 340), (0, T)):
+            got = layer(h[lo:hi].to(dev)).double().cpu()
+            d = got - ref[lo:hi]
+            bad = (d.abs().max(-1).values > 3e-2 * ref.abs().max()).nonzero().flatten().tolist()
+            assert len(bad) <= (hi - lo) // 100, f"{E} + {ident} experts, tokens {lo}:{hi}: rows {bad[:5]} differ (a tipped choice is rare)"
+
+
 def test_the_correction_moves_the_choice_not_the_weights_and_identity_returns_the_input(backend):
     dev = device_of(backend)
     ops = make_ops(backend, torch.float32, dev)
